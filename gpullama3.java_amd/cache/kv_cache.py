@@ -43,6 +43,9 @@ class KVNeed:
     v_head_dim: Optional[int] = None         # None: as the keys'
     values: bool = True                      # False: no second array (``layer_kv`` then gives (keys, None))
     keep_first: int = 0                      # with a window: the sequence's first positions that stay visible (and stored)
+    v_heads: Optional[int] = None            # value heads where they are fewer than the key heads (several score maps
+                                             # over the same values); None: as many
+    chunk: Optional[int] = None              # n: a query sees the keys of its own run of n positions only (no window then)
 
     @property
     def value_dim(self):
@@ -85,7 +88,7 @@ class CacheGroup:
         self.k = torch.zeros((n, n_pages, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
         # values lie transposed inside a page: the order in which the attention kernels' second
         # product reads them (and both in tiles, see layout.py)
-        self.v = (torch.zeros((n, n_pages, need.n_kv_heads, need.value_dim, page_size), dtype=dtype, device=device)
+        self.v = (torch.zeros((n, n_pages, need.v_heads or need.n_kv_heads, need.value_dim, page_size), dtype=dtype, device=device)
                   if need.values else None)
         self.table = None            # [n_slots + 1, pages of the longest sequence] int32 on the device
         self.table_host = None       # the same on the host (numpy), the copy that the bookkeeping writes
@@ -121,7 +124,7 @@ class Cache:
                 self.group_of[e] = (len(self.groups), i)
             self.groups.append(g)
         self.slots = SlotTable(n_slots, len(self.groups))
-        self._windowed = any(g.need.window for g in self.groups)
+        self._windowed = any(g.need.window or g.need.chunk for g in self.groups)
         self.sink_slot = n_slots                             # the row of padded entries: no sequence's
         for g in self.groups:
             g.table_host = np.zeros((n_slots + 1, self.max_pages_per_seq), dtype=np.int32)
@@ -197,11 +200,14 @@ class Cache:
         page, which nobody reads."""
         self.slots.length[s] += n
         for g, group in enumerate(self.groups):
-            window = group.need.window
-            if not window:
+            window, chunk = group.need.window, getattr(group.need, "chunk", None)
+            if not window and not chunk:
                 continue
             pages = self.slots.pages[s][g]
-            first_seen = max(0, self.slots.length[s] + 1 - window) // self.page_size
+            if chunk:      # the next token, at position ``length``, reads the keys from its chunk's first position on
+                first_seen = (self.slots.length[s] // chunk) * chunk // self.page_size
+            else:
+                first_seen = max(0, self.slots.length[s] + 1 - window) // self.page_size
             # (the pages of the first positions that every later token still sees are held to the sequence's end)
             kept = -(-int(getattr(group.need, "keep_first", 0) or 0) // self.page_size)
             gone = [i for i in range(kept, min(first_seen, len(pages))) if pages[i]]

@@ -6,9 +6,10 @@ from .specs import (AttentionSpec, BlockSpec, DistanceBias, GatedDeltaSpec, Gate
 from .llama import LlamaConfiguration
 from .melizen import MelizenConfiguration
 from .nodupel import NodupelConfiguration
+from .nolatar import NolatarConfiguration
 
 __all__ = ["ConfigError", "config_from_dict", "load_config", "register_architecture",
            "registered_architectures", "AttentionSpec", "BlockSpec", "GatedFeedForwardSpec",
            "Llama3RopeScaling", "ModelSpec", "NormSpec", "RotarySpec", "Run", "LlamaConfiguration", "DistanceBias", "GatedDeltaSpec", "Inject",
            "MelizenConfiguration", "NodupelConfiguration", "LinearRopeScaling", "MinGRUSpec", "PairEmbedding", "Remix",
-           "SideBySideSpec", "TimeMixSpec"]
+           "SideBySideSpec", "TimeMixSpec", "NolatarConfiguration"]

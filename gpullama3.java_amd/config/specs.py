@@ -50,6 +50,26 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """``(x - mean(x)) / sqrt(var(x) + eps) * w + b`` with the variance as the mean of the squared deviations."""
+    kind: str = "layernorm"
+    dim: int = 0
+    eps: float = 1e-5
+    names: dict = field(default_factory=dict)     # "weight", "bias" -> stored names
+
+
+@dataclass(frozen=True)
+class Differential:
+    """Differential attention: every head has two score maps (queries and keys of their own, the same values); the
+    head's output is ``a1 - lambda * a2`` divided by its root mean square (``norm_eps`` inside the root) times
+    ``1 - offset``, with ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + offset`` from four stored vectors of the keys'
+    size (names ``lambda_q1``, ``lambda_k1``, ``lambda_q2``, ``lambda_k2`` of the attention). The stored rows of q and
+    k lie head by head as [map 1, map 2]."""
+    offset: float = 0.0
+    norm_eps: float = 1e-5
+
+
+@dataclass(frozen=True)
 class DistanceBias:
     """A bias on the attention scores that grows with the distance: head h of H takes
     ``slope_h * (i - j)`` off the score of query i and key j, ``slope_h = base ** (-exponent * (h + 1) / H)``."""
@@ -82,6 +102,12 @@ class AttentionSpec:
     value_position: Optional[RotarySpec] = None   # values are rotated by their own position before they are cached (over the
                                       # whole value head), and each head's output is turned back by the query's position
     out_mult: float = 1.0             # a constant that the mixer's output is multiplied by
+    qk_norm_eps: Optional[float] = None   # queries and keys are divided by their root mean square per head (this eps
+                                      # inside the root) and multiplied by the stored [head_dim] weights ``q_norm`` /
+                                      # ``k_norm`` (shared by the heads) before the rotation; None: no such norm
+    chunk: Optional[int] = None       # n: query i sees key j <= i only if i // n == j // n (chunks count from position 0)
+    differential: Optional[Differential] = None
+    # (no ``k`` among ``names``: the mixer has no keys and values of its own and only ever reads another entry's)
     # (a name ``head_gate`` among ``names``: a stored [n_heads, hidden] matrix; head h's output is multiplied by
     # sigmoid of its row's product with the mixer's input, before the output projection)
 
@@ -125,6 +151,46 @@ class SideBySideSpec:
     weight: float = 0.5
     names: dict = field(default_factory=dict)     # "left_norm", "right_norm": the stored [hidden] weights
     out_mult: float = 1.0
+    normalised: bool = True           # False: the mixer's output is the plain sum of the sides' outputs (each side
+                                      # carries its own factor as its ``out_mult``); no norms, no weights
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head and no softmax (``parts/retention.py``): per head a matrix
+    S [key_dim, value_dim] in 32-bit, ``S <- decay_h S + k v^T`` with k times ``key_dim ** -0.5``, ``o = S^T q``; q and
+    k are rotated like an attention's. Each head's read-out is divided by its root mean square, the heads together are
+    multiplied by silu of a gate projection, then the output projection."""
+    kind: str = "retention"
+    hidden: int = 0
+    n_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    decay: tuple = ()                 # one factor per head
+    position: Optional[RotarySpec] = None
+    norm_eps: float = 1e-5
+    names: dict = field(default_factory=dict)     # "q", "k", "v", "g", "o"
+    out_mult: float = 1.0
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A selective state space with a scalar decay per head and token (``parts/state_space.py``): one projection gives
+    [z | x | B | C | dt]; x, B and C pass a causal convolution of ``conv_taps`` taps per channel and silu; per head
+    (``n_heads`` heads of ``head_dim`` share ``n_groups`` B and C of ``state_dim``) ``S <- exp(-exp(A_log) dt) S + dt B
+    x^T``, ``y = S^T C + D x`` with ``dt = softplus(dt + dt_bias)``; y times silu(z), divided by its root mean square in
+    ``norm_groups`` equal parts, times a weight, then the output projection."""
+    kind: str = "state_space"
+    hidden: int = 0
+    n_heads: int = 0
+    head_dim: int = 0
+    n_groups: int = 1
+    state_dim: int = 0
+    conv_taps: int = 4
+    norm_groups: int = 1
+    norm_eps: float = 1e-5
+    names: dict = field(default_factory=dict)     # "in", "conv", "conv_bias", "dt_bias", "A_log", "D", "norm", "o"
+    out_mult: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -162,9 +228,35 @@ class GatedFeedForwardSpec:
 
 
 @dataclass(frozen=True)
+class ExpertSpec:
+    """One small feed-forward without a gate: ``down(act(up h))``; ``activation`` "gelu" (the erf form), "gelu_tanh"
+    or "silu"."""
+    intermediate: int = 0
+    activation: str = "gelu"
+
+
+@dataclass(frozen=True)
+class RoutedFeedForwardSpec:
+    """A mixture of experts (``parts/routed.py``): router logits in 32-bit, the ``top`` largest choose a token's
+    experts, their weights are the softmax over the chosen logits alone; ``shared`` (an ``ExpertSpec`` or None) runs
+    for every token and is added. Stored names: ``router`` [experts, hidden]; ``expert_up`` / ``expert_down`` are
+    patterns with ``{e}`` for the expert's number; ``shared_up`` / ``shared_down``."""
+    kind: str = "routed"
+    hidden: int = 0
+    n_experts: int = 0
+    top: int = 1
+    expert: ExpertSpec = None
+    shared: Optional[ExpertSpec] = None
+    names: dict = field(default_factory=dict)
+    out_mult: float = 1.0
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: how norm, mixer and feed-forward are arranged is ``kind``. "prenorm": x += mixer(norm(x));
-    x += ffn(norm(x)). "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h) (one norm, ``ffn_norm`` is None)."""
+    x += ffn(norm(x)). "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h) (one norm, ``ffn_norm`` is None).
+    "outnorm": x += mixer_norm(mixer(x)); x += ffn_norm(ffn(x)): the sublayers read the rows themselves, the norms
+    stand behind them."""
     kind: str = "prenorm"
     mixer_norm: object = None
     mixer: object = None

@@ -16,7 +16,11 @@
 // query head; and a sink, a key that every query sees with the score `sink` and whose value is
 // zero, so that the weights of the real keys sum to less than one: exp(s_j) / (exp(sink) + sum exp(s)).
 // The sink is the running softmax's starting point (maximum = sink, sum = 1). And a window that keeps a sequence's
-// first keys visible (keep_first): query p sees key j <= p if p - j < window or j < keep_first.
+// first keys visible (keep_first): query p sees key j <= p if p - j < window or j < keep_first. A chunked mask (chunk > 0, no
+// window): query p sees key j <= p only if j / chunk == p / chunk. And fewer value heads than key heads (n_v): several
+// score maps over the same values. With maps = n_kv / n_v, query heads and key heads lie head by head as [map 0, map 1,
+// ...]: query head h is map h % maps of head h / maps, which reads key head g * maps + h % maps and value head g, g the
+// head's group.
 #include "common.h"
 
 #define ATT_MAX_HS 256
@@ -26,14 +30,17 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, T* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
-    int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
+    int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink, int keep_first,
+    int chunk, int n_v) {
   __shared__ float qs[ATT_MAX_HS];
   __shared__ float ps[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = positions[t];
-  const int c = h / (n_heads / n_kv);
+  const int maps = n_kv / n_v;
+  const int cv = (h / maps) / ((n_heads / maps) / n_v);
+  const int c = cv * maps + h % maps;
   const int* bt = block_table + (long)seq_of_token[t] * table_stride;
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = chunk > 0 ? (p / chunk) * chunk : (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const T* qp = q + (long)t * q_stride + (long)h * head_dim;
   for (int i = lane; i < head_dim; i += 64) qs[i] = to_f32<T>(qp[i]);
   __syncthreads();
@@ -69,7 +76,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     for (int j = 0; j < n_valid; ++j) {
       const int kj = base + j;
       // values lie transposed in a page: [head_dim][position in page], in tiles
-      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * v_head_dim;
+      const T* vp = v_cache + ((long)bt[kj / page_size] * n_v + cv) * page_size * v_head_dim;
       const int in_page = kj % page_size;
       const float w = ps[j];
 #pragma unroll
@@ -93,7 +100,8 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
                                      const int* positions, const int* seq_of_token, const int* block_table,
                                      int table_stride, void* out, long out_stride, int n_tokens, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int v_head_dim,
-                                     const float* slopes, int has_sink, float sink, int keep_first, hipStream_t stream) {
+                                     const float* slopes, int has_sink, float sink, int keep_first, int chunk, int n_v,
+                                     hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
               "gl3_attention_generic: null argument");
@@ -106,6 +114,9 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
   GL3_REQUIRE(n_heads <= 65535, "gl3_attention_generic: %d heads exceed the grid", n_heads);
   GL3_REQUIRE(page_size > 0 && table_stride > 0, "gl3_attention_generic: bad paging");
   GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_generic: %d kept first keys without a window", keep_first);
+  GL3_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "gl3_attention_generic: a chunked mask has no window");
+  GL3_REQUIRE(n_v > 0 && n_kv % n_v == 0 && n_heads % (n_kv / n_v) == 0 && (n_heads / (n_kv / n_v)) % n_v == 0,
+              "gl3_attention_generic: %d heads, %d key heads, %d value heads", n_heads, n_kv, n_v);
   GL3_REQUIRE(page_size % 32 == 0 && head_dim % 16 == 0,
               "gl3_attention_generic: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16", page_size,
               head_dim);
@@ -114,12 +125,12 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
     attention_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, positions, seq_of_token, block_table,
         table_stride, (float*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink,
-        sink, keep_first);
+        sink, keep_first, chunk, n_v);
   else if (dtype == GL3_BF16)
     attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,
         block_table, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale,
-        slopes, has_sink, sink, keep_first);
+        slopes, has_sink, sink, keep_first, chunk, n_v);
   else GL3_REQUIRE(false, "gl3_attention_generic: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;

@@ -644,3 +644,97 @@ extern "C" int gl3_residual_inject(float* x, const float* rows, const float* vec
   GL3_LAUNCH_CHECK();
   return 0;
 }
+
+// ----------------------------------------------------------------- layer norm
+// (y - mean(y)) / sqrt(var(y) + eps) * w + b with the variance as the mean of the squared deviations (two passes over
+// the row: the mean first). One block a row; the order of the sums depends on d and the block's size alone.
+//   gl3_layernorm:      out[r] = LN(x[rows ? rows[r] : r]) in the activations' type.
+//   gl3_layernorm_add:  x[t] += LN(y[t]) (x and y float), and cast[t] = x[t] in the activations' type where `cast`
+//                       is given: what the sublayer that reads the rows next takes as its input.
+__device__ __forceinline__ void layernorm_stats(const float* __restrict__ y, int d, float eps, float* scratch, float* mean_out,
+                                                float* inv_out) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) s += y[i];
+  const float mean = block_sum(s, scratch) / (float)d;
+  float v = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float dlt = y[i] - mean;
+    v += dlt * dlt;
+  }
+  *mean_out = mean;
+  *inv_out = 1.0f / sqrtf(block_sum(v, scratch) / (float)d + eps);
+}
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                                          const float* __restrict__ w, const float* __restrict__ b,
+                                                          TO* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[16];
+  const long r = blockIdx.x;
+  const float* y = x + (long)(rows ? rows[r] : r) * d;
+  float mean, inv;
+  layernorm_stats(y, d, eps, scratch, &mean, &inv);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) out[r * d + i] = from_f32<TO>((y[i] - mean) * inv * w[i] + b[i]);
+}
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void layernorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                              const float* __restrict__ w, const float* __restrict__ b,
+                                                              int d, float eps, TO* __restrict__ cast) {
+  __shared__ float scratch[16];
+  const long t = blockIdx.x;
+  const float* yr = y + t * d;
+  float mean, inv;
+  layernorm_stats(yr, d, eps, scratch, &mean, &inv);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float v = x[t * d + i] + ((yr[i] - mean) * inv * w[i] + b[i]);
+    x[t * d + i] = v;
+    if (cast) cast[t * d + i] = from_f32<TO>(v);
+  }
+}
+
+static int layernorm_threads(int d) { return d >= 1024 ? 1024 : ((d + 63) / 64) * 64; }
+
+extern "C" int gl3_layernorm(const float* x, const int* rows, const float* w, const float* b, void* out, int out_dtype,
+                             int n_rows, int d, float eps, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(x && w && b && out && n_rows > 0 && d > 0, "gl3_layernorm: bad arguments (rows=%d d=%d)", n_rows, d);
+  const dim3 grid(n_rows), block(layernorm_threads(d));
+  if (out_dtype == GL3_F32) layernorm_kernel<float><<<grid, block, 0, stream>>>(x, rows, w, b, (float*)out, d, eps);
+  else if (out_dtype == GL3_BF16) layernorm_kernel<bf16_t><<<grid, block, 0, stream>>>(x, rows, w, b, (bf16_t*)out, d, eps);
+  else GL3_REQUIRE(false, "gl3_layernorm: unknown dtype %d", out_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int gl3_layernorm_add(float* x, const float* y, const float* w, const float* b, int n_rows, int d, float eps,
+                                 void* cast, int cast_dtype, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(x && y && w && b && n_rows > 0 && d > 0, "gl3_layernorm_add: bad arguments (rows=%d d=%d)", n_rows, d);
+  const dim3 grid(n_rows), block(layernorm_threads(d));
+  if (!cast || cast_dtype == GL3_F32)
+    layernorm_add_kernel<float><<<grid, block, 0, stream>>>(x, y, w, b, d, eps, (float*)cast);
+  else if (cast_dtype == GL3_BF16)
+    layernorm_add_kernel<bf16_t><<<grid, block, 0, stream>>>(x, y, w, b, d, eps, (bf16_t*)cast);
+  else GL3_REQUIRE(false, "gl3_layernorm_add: unknown dtype %d", cast_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- float rows in the activations' type
+template <typename TO>
+__global__ void cast_rows_kernel(const float* __restrict__ in, TO* __restrict__ out, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<TO>(in[i]);
+}
+
+extern "C" int gl3_cast_rows(const float* in, void* out, int out_dtype, long n, hipStream_t stream) {
+  if (n == 0) return 0;
+  GL3_REQUIRE(in && out && n > 0 && (n + 255) / 256 < (1L << 31), "gl3_cast_rows: bad arguments");
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (out_dtype == GL3_F32) cast_rows_kernel<float><<<grid, block, 0, stream>>>(in, (float*)out, n);
+  else if (out_dtype == GL3_BF16) cast_rows_kernel<bf16_t><<<grid, block, 0, stream>>>(in, (bf16_t*)out, n);
+  else GL3_REQUIRE(false, "gl3_cast_rows: unknown dtype %d", out_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

@@ -57,10 +57,20 @@ def _declare(lib):
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, F, F, P, P],
-        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
         "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
         "gl3_concat_rows": [P, P, P, I, I, I, P],
-        "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P],
+        "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P, P, F, P],
+        "gl3_diff_combine": [P, L, P, L, I, I, I, I, I, F, F, F, P],
+        "gl3_layernorm": [P, P, P, P, P, I, I, I, F, P],
+        "gl3_layernorm_add": [P, P, P, P, I, I, F, P, I, P],
+        "gl3_cast_rows": [P, P, I, L, P],
+        "gl3_ssm_prep": [P, L, I, I, I, I, I, I, P, P, I, P, P, P, L, L, P, P, P, P, P, P],
+        "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P],
+        "gl3_group_norm_gate": [P, P, L, I, P, I, P, L, I, P, F, I, I, I, I, P, I, P],
+        "gl3_route": [P, I, I, I, P, P, P, P, P],
+        "gl3_expert_gemm": [P, I, L, I, P, I, I, I, I, P, P, I, P, I, L, I, I, P],
+        "gl3_route_combine": [P, P, I, I, I, P, I, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
@@ -164,7 +174,7 @@ def _ptr(t):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
 
-def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who, v_head_dim=None):
+def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who, v_head_dim=None, n_v=None):
     """Keys [pages, kv heads, page, head_dim]; values transposed [pages, kv heads, head_dim, page]; inside a
     page both lie in the kernels' tiles (``cache/layout.py``), which needs pages of a multiple of 32 positions
     and heads of a multiple of 16 elements. ``v_head_dim``: the values' size where a kernel takes another than the keys'."""
@@ -172,7 +182,7 @@ def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who, v_head_dim=No
     if vd % 16:
         raise KernelError(f"{who}: values of {vd} elements are not a multiple of 16")
     if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim)
-            or tuple(v_cache.shape) != (k_cache.shape[0], n_kv, vd, page_size)):
+            or tuple(v_cache.shape) != (k_cache.shape[0], n_kv if n_v is None else n_v, vd, page_size)):
         raise KernelError(f"{who}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for kv {n_kv} "
                           f"page {page_size} hs {head_dim}")
     if page_size % 32 or head_dim % 16:
@@ -390,11 +400,14 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu", act_limit
 
 
 def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None, keep_first=0):
+                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None, keep_first=0, chunk=0, n_v_heads=None):
     """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries. ``v_head_dim``: the values'
     size where it is not the keys'; ``slopes``: float32 [H], score - slopes[h] * distance; ``sink``: the score of a
     key without a value that every query sees (None: no such key); ``keep_first``: with a window, the sequence's
-    first keys that stay visible to every later query."""
+    first keys that stay visible to every later query; ``chunk``: n > 0: query i sees key j <= i only if
+    i // n == j // n (no window then); ``n_v_heads``: value heads where they are fewer than the key heads: several
+    score maps over the same values, ``maps = n_kv / n_v_heads``; query and key heads then lie head by head as
+    [map 0, map 1, ...], and map m of a head reads key head ``g * maps + m`` and value head g of the head's group."""
     _dev(q, "q", contiguous=False); _dev(out, "out", contiguous=False)
     _dev(k_cache, "k_cache", q.dtype); _dev(v_cache, "v_cache", q.dtype)
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
@@ -405,9 +418,12 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     vd = head_dim if v_head_dim is None else int(v_head_dim)
     if out.shape != (T, n_heads * vd) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
-    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", vd)
+    n_v = n_kv if n_v_heads is None else int(n_v_heads)
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", vd, n_v)
     if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
+    if chunk and window:
+        raise KernelError("attention: a chunked mask has no window")
     if slopes is not None:
         _dev(slopes, "slopes", torch.float32)
         if slopes.shape != (n_heads,):
@@ -416,7 +432,7 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
         int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0),
-        int(keep_first or 0) if window else 0, _stream()),
+        int(keep_first or 0) if window else 0, int(chunk or 0), n_v, _stream()),
         "attention_generic")
 
 
@@ -480,13 +496,17 @@ def concat_rows(a, b, out):
            "concat_rows")
 
 
-def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, gate_col=0, cache=None):
+def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, gate_col=0, cache=None, norms=None,
+                 norm_eps=0.0):
     """Runs of heads inside ``rows`` [T, ld] turned in place by the tokens' positions. ``runs``: up to three of
     ``(first column, heads, head_dim, rot_dim, cos, sin)`` with tables [positions, rot_dim / 2] float32 (None, None: not
     rotated). ``back``: by minus the angle. ``gate`` (one run): rows [T, *] of the same dtype whose column
     ``gate_col + h`` holds head h's gate; every element of the head is multiplied by its sigmoid. ``cache``:
     ``(k_cache, v_cache, table_rows, block_table, page_size)``; the runs are then queries, keys and values, and keys and
-    values also go to the tokens' places in one layer's paged cache."""
+    values also go to the tokens' places in one layer's paged cache (the values may have fewer heads than the keys).
+    ``norms``: per run None or ``(weight float32 [head_dim], n)``: the run's heads are first divided by their root
+    mean square over their first n elements (``norm_eps`` inside the root; what lies behind them must be zeros) and
+    multiplied by the weight."""
     _dev(rows, "rows", contiguous=False); _dev(positions, "positions", torch.int32)
     T = rows.shape[0]
     if rows.dim() != 2 or rows.stride(1) != 1 or positions.numel() != T or not 1 <= len(runs) <= 3:
@@ -513,13 +533,222 @@ def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, g
         kc, vc, trows, table, page = cache
         _dev(trows, "table_rows", torch.int32); _dev(table, "block_table", torch.int32)
         _dev(kc, "k_cache", rows.dtype); _dev(vc, "v_cache", rows.dtype)
-        if n != 3 or runs[1][1] != runs[2][1] or trows.numel() != T or table.dim() != 2:
+        if n != 3 or trows.numel() != T or table.dim() != 2:
             raise KernelError("rotate_heads: a cache write takes queries, keys and values and a table row per token")
-        _check_cache(kc, vc, runs[1][1], page, runs[1][2], "rotate_heads", runs[2][2])
+        _check_cache(kc, vc, runs[1][1], page, runs[1][2], "rotate_heads", runs[2][2], runs[2][1])
         stride = table.shape[1]
+    norm_ws = norm_dims = None
+    if norms is not None and any(x is not None for x in norms):
+        if len(norms) != n:
+            raise KernelError(f"rotate_heads: {len(norms)} norms for {n} runs")
+        for (w, nd), r in zip([x if x is not None else (None, 0) for x in norms], runs):
+            if w is not None:
+                _dev(w, "norm weight", torch.float32)
+                if w.shape != (r[2],) or not 0 < nd <= r[2]:
+                    raise KernelError(f"rotate_heads: a norm weight {tuple(w.shape)} over {nd} of a head's {r[2]} elements")
+        norm_ws = (c_void_p * n)(*[x[0].data_ptr() if x is not None else None for x in norms])
+        norm_dims = (c_int * n)(*[int(x[1]) if x is not None else 0 for x in norms])
     _check(library().gl3_rotate_heads(_ptr(rows), _code(rows, "rows"), rows.stride(0), _ptr(positions), T, *ints, *tabs, n,
                                       int(bool(adjacent)), int(bool(back)), _ptr(gate), gate_ld, int(gate_col), _ptr(kc),
-                                      _ptr(vc), _ptr(trows), _ptr(table), stride, int(page), _stream()), "rotate_heads")
+                                      _ptr(vc), _ptr(trows), _ptr(table), stride, int(page), norm_ws, norm_dims,
+                                      float(norm_eps), _stream()), "rotate_heads")
+
+
+def diff_combine(att, out, H, D, dim, lam, eps, mult):
+    """``att`` [T, 2 H D]: head by head the output under the first score map and under the second; ``out`` [T, H D] =
+    (a1 - lam * a2) / rms over the head's first ``dim`` elements (what lies behind them holds zeros) * mult."""
+    _dev(att, "att", contiguous=False); _dev(out, "out", att.dtype, contiguous=False)
+    T = att.shape[0]
+    if att.dim() != 2 or att.stride(1) != 1 or att.shape[1] < 2 * H * D or out.shape != (T, H * D) or out.stride(1) != 1:
+        raise KernelError(f"diff_combine: {tuple(att.shape)} -> {tuple(out.shape)} for {H} heads of {D}")
+    _check(library().gl3_diff_combine(_ptr(att), att.stride(0), _ptr(out), out.stride(0), _code(att, "att"), T, int(H), int(D),
+                                      int(dim), float(lam), float(eps), float(mult), _stream()), "diff_combine")
+
+
+def layernorm(x, weight, bias, out, eps, rows=None):
+    """out[r] = layer norm of x[rows[r]] (of x[r] without ``rows``) with float32 weight and bias."""
+    _dev(x, "x", torch.float32); _dev(weight, "weight", torch.float32); _dev(bias, "bias", torch.float32); _dev(out, "out")
+    d = x.shape[1]
+    n = x.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+    if x.dim() != 2 or weight.shape != (d,) or bias.shape != (d,) or out.shape != (n, d):
+        raise KernelError(f"layernorm: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(bias), _ptr(out), _code(out, "out"), n, d,
+                                   float(eps), _stream()), "layernorm")
+
+
+def layernorm_add(x, y, weight, bias, eps, cast=None):
+    """x += layer norm of y, row by row (both float32); ``cast`` (same shape, the activations' type) receives the new
+    rows of x."""
+    _dev(x, "x", torch.float32); _dev(y, "y", torch.float32)
+    _dev(weight, "weight", torch.float32); _dev(bias, "bias", torch.float32)
+    T, d = x.shape
+    if x.dim() != 2 or y.shape != (T, d) or weight.shape != (d,) or bias.shape != (d,):
+        raise KernelError(f"layernorm_add: x {tuple(x.shape)}, y {tuple(y.shape)}, weight {tuple(weight.shape)}")
+    if cast is not None:
+        _dev(cast, "cast")
+        if cast.shape != (T, d):
+            raise KernelError(f"layernorm_add: cast {tuple(cast.shape)}")
+    _check(library().gl3_layernorm_add(_ptr(x), _ptr(y), _ptr(weight), _ptr(bias), T, d, float(eps), _ptr(cast),
+                                       _code(cast, "cast") if cast is not None else F32, _stream()), "layernorm_add")
+
+
+def cast_rows(x, out):
+    """``out`` = the float32 ``x`` in out's type."""
+    _dev(x, "x", torch.float32); _dev(out, "out")
+    if out.shape != x.shape:
+        raise KernelError(f"cast_rows: {tuple(x.shape)} -> {tuple(out.shape)}")
+    _check(library().gl3_cast_rows(_ptr(x), _ptr(out), _code(out, "out"), x.numel(), _stream()), "cast_rows")
+
+
+def _f32_rows(t, name, cols):
+    _dev(t, name, torch.float32, contiguous=False)
+    if t.dim() != 2 or t.stride(1) != 1 or t.shape[1] < cols:
+        raise KernelError(f"{name}: rows {tuple(t.shape)} hold fewer than {cols} columns")
+    return t
+
+
+def _state_area(state, state_off, need, who):
+    _dev(state, "state", torch.float32, contiguous=False)
+    if state.dim() != 2 or state.stride(1) != 1 or state_off < 0 or state_off + need > state.shape[1]:
+        raise KernelError(f"{who}: a state of {tuple(state.shape)} for {need} floats from {state_off}")
+
+
+def ssm_prep(proj, col_x, channels, col_dt, heads, conv_w, conv_b, A_log, dt_bias, state, state_off, cu_seqlens,
+             seq_of_token, slot_ids, act, ab):
+    """The state space's short convolution with silu over ``channels`` columns of ``proj`` [T, ld] float32 from
+    ``col_x`` on (``conv_w`` [channels, taps], the last tap the current token's; the sequences' last taps - 1 inputs
+    live in ``state`` [slots, *] from ``state_off`` on and move on) -> ``act`` [T, channels]; and per head the decay
+    and the step size from column ``col_dt`` on -> ``ab`` [T, 2 heads] = (exp(-exp(A_log) dt), dt), dt = softplus(. + dt_bias)."""
+    T = proj.shape[0]
+    _f32_rows(proj, "proj", max(col_x + channels, col_dt + heads))
+    taps = conv_w.shape[1]
+    for t, name, shape in ((conv_w, "conv_w", (channels, taps)), (A_log, "A_log", (heads,)), (dt_bias, "dt_bias", (heads,)),
+                           (act, "act", (T, channels)), (ab, "ab", (T, 2 * heads))):
+        _dev(t, name, torch.float32)
+        if tuple(t.shape) != shape:
+            raise KernelError(f"ssm_prep: {name} {tuple(t.shape)}, expected {shape}")
+    if conv_b is not None:
+        _dev(conv_b, "conv_b", torch.float32)
+        if conv_b.shape != (channels,):
+            raise KernelError(f"ssm_prep: conv_b {tuple(conv_b.shape)}")
+    _state_area(state, state_off, (taps - 1) * channels, "ssm_prep")
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
+    B = cu_seqlens.numel() - 1
+    if seq_of_token.numel() != T or slot_ids.numel() < B:
+        raise KernelError("ssm_prep: seq_of_token / slot_ids shapes")
+    _check(library().gl3_ssm_prep(_ptr(proj), proj.stride(0), T, B, int(col_x), int(channels), int(col_dt), int(heads),
+                                  _ptr(conv_w), _ptr(conv_b), taps, _ptr(A_log), _ptr(dt_bias), _ptr(state), state.stride(0),
+                                  int(state_off), _ptr(cu_seqlens), _ptr(seq_of_token), _ptr(slot_ids), _ptr(act), _ptr(ab),
+                                  _stream()), "ssm_prep")
+
+
+def decay_scan(q, col_q, k, col_k, v, col_v, state, state_off, cu_seqlens, slot_ids, out, H, heads_per_group, N, P,
+               a_tok=None, b_tok=None, a_head=None, b_const=1.0):
+    """Per (sequence, head) ``S <- a S + b k v^T`` and ``o = S^T q`` token by token, S [N, P] float32 in ``state``
+    [slots, *] from ``state_off + h N P`` on. q and k: float32 rows whose group g (``heads_per_group`` heads share one)
+    starts at column ``col + g N``; v: head h at ``col_v + h P``. a and b: per token and head (``a_tok``, ``b_tok``,
+    columns h of rows of the same stride) or per head (``a_head`` [H]) / one number (``b_const``). ``out`` [T, H P]."""
+    groups = H // heads_per_group
+    _f32_rows(q, "q", col_q + groups * N); _f32_rows(k, "k", col_k + groups * N); _f32_rows(v, "v", col_v + H * P)
+    _dev(out, "out", torch.float32)
+    T = q.shape[0]
+    if k.shape[0] != T or v.shape[0] != T or out.shape != (T, H * P):
+        raise KernelError(f"decay_scan: rows {q.shape[0]}, {k.shape[0]}, {v.shape[0]}; out {tuple(out.shape)}")
+    ld_ab = 0
+    for t, name in ((a_tok, "a_tok"), (b_tok, "b_tok")):
+        if t is not None:
+            _f32_rows(t, name, H)
+            if t.shape[0] != T or (ld_ab and t.stride(0) != ld_ab):
+                raise KernelError(f"decay_scan: {name} {tuple(t.shape)}")
+            ld_ab = t.stride(0)
+    if a_tok is None:
+        _dev(a_head, "a_head", torch.float32)
+        if a_head.shape != (H,):
+            raise KernelError(f"decay_scan: a_head {tuple(a_head.shape)}")
+    _state_area(state, state_off, H * N * P, "decay_scan")
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
+    B = cu_seqlens.numel() - 1
+    _check(library().gl3_decay_scan(_ptr(q), q.stride(0), int(col_q), _ptr(k), k.stride(0), int(col_k), _ptr(v), v.stride(0),
+                                    int(col_v), _ptr(a_tok), _ptr(b_tok), ld_ab, _ptr(a_head), float(b_const), _ptr(state),
+                                    state.stride(0), int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
+                                    out.stride(0), B, int(H), int(heads_per_group), int(N), int(P), _stream()), "decay_scan")
+
+
+def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=False, skip=None):
+    """``o`` [T, C] float32 (+ ``skip = (rows, col, d [heads], head_dim)``: d[h] times the rows' columns), times silu of
+    the gate columns (``gate`` rows float32 from ``col_g``) before (``gate_first``) or after being divided by its root
+    mean square over every ``gsize`` channels; times ``weight`` [C]. ``out`` [T, C] in the activations' type."""
+    _dev(o, "o", torch.float32); _dev(out, "out")
+    T, C = o.shape
+    _f32_rows(gate, "gate", col_g + C)
+    if out.shape != (T, C) or gate.shape[0] != T or C % gsize:
+        raise KernelError(f"group_norm_gate: o {tuple(o.shape)}, out {tuple(out.shape)}, groups of {gsize}")
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
+        if weight.shape != (C,):
+            raise KernelError(f"group_norm_gate: weight {tuple(weight.shape)}")
+    sx = sd = None
+    ld_x = col_x = hd = 0
+    if skip is not None:
+        sx, col_x, sd, hd = skip
+        _f32_rows(sx, "skip rows", col_x + C); _dev(sd, "skip factors", torch.float32)
+        if sx.shape[0] != T or C % hd or sd.shape != (C // hd,):
+            raise KernelError(f"group_norm_gate: skip rows {tuple(sx.shape)}, factors {tuple(sd.shape)}")
+        ld_x = sx.stride(0)
+    _check(library().gl3_group_norm_gate(_ptr(o), _ptr(sx), ld_x, int(col_x), _ptr(sd), int(hd), _ptr(gate), gate.stride(0),
+                                         int(col_g), _ptr(weight), float(eps), int(bool(gate_first)), T, C, int(gsize),
+                                         _ptr(out), _code(out, "out"), _stream()), "group_norm_gate")
+
+
+EXPERT_ACTIVATIONS = {None: 0, "gelu": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def route(logits, top, idx, wts, offsets, pairs):
+    """Router logits [T, E] float32 -> the ``top`` largest per token (``idx`` [T, top] int32, the lower number wins a
+    tie) with the softmax over them alone (``wts`` [T, top]); and the (token, choice) pairs ordered by expert:
+    ``offsets`` [E + 1] int32, ``pairs`` [T top] int32 (pair t * top + j)."""
+    _dev(logits, "logits", torch.float32)
+    T, E = logits.shape
+    for t, name, shape, dt in ((idx, "idx", (T, top), torch.int32), (wts, "wts", (T, top), torch.float32),
+                               (offsets, "offsets", (E + 1,), torch.int32), (pairs, "pairs", (T * top,), torch.int32)):
+        _dev(t, name, dt)
+        if tuple(t.shape) != shape:
+            raise KernelError(f"route: {name} {tuple(t.shape)}, expected {shape}")
+    _check(library().gl3_route(_ptr(logits), T, E, int(top), _ptr(idx), _ptr(wts), _ptr(offsets), _ptr(pairs), _stream()), "route")
+
+
+def expert_gemm(a, w, out, act=None, offsets=None, pairs=None, a_div=1, mfma=True):
+    """``out[p] = act(w[e] @ a[p // a_div])`` for every pair p of expert e's run (``offsets``, ``pairs`` of ``route``);
+    without them ``w`` is one expert [1, N, K] that takes every row of ``a`` in its own order. ``w`` [E, N, K];
+    ``out`` [pairs, N] in bfloat16 or float32."""
+    _dev(a, "a", contiguous=False); _dev(w, "w", a.dtype); _dev(out, "out", contiguous=False)
+    if w.dim() != 3 or a.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1 or a.shape[1] != w.shape[2] or out.shape[1] != w.shape[1]:
+        raise KernelError(f"expert_gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    E, N, K = w.shape
+    n_rows = out.shape[0]
+    if offsets is not None:
+        _dev(offsets, "offsets", torch.int32); _dev(pairs, "pairs", torch.int32)
+        if offsets.numel() != E + 1 or pairs.numel() != n_rows or a.shape[0] * a_div < n_rows:
+            raise KernelError(f"expert_gemm: {offsets.numel()} offsets, {pairs.numel()} pairs, {a.shape[0]} rows x {a_div}")
+    elif E != 1 or a.shape[0] != n_rows or a_div != 1:
+        raise KernelError("expert_gemm: without runs one expert takes every row")
+    if act not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"expert_gemm: activation {act!r} is not built ({sorted(k for k in EXPERT_ACTIVATIONS if k)})")
+    _check(library().gl3_expert_gemm(_ptr(a), _code(a, "a"), a.stride(0), int(a_div), _ptr(w), _code(w, "w"), E, N, K,
+                                     _ptr(offsets), _ptr(pairs), n_rows, _ptr(out), _code(out, "out"), out.stride(0),
+                                     EXPERT_ACTIVATIONS[act], int(bool(mfma)), _stream()), "expert_gemm")
+
+
+def route_combine(y, wts, out, accumulate=False):
+    """``out[t]`` (+)= sum over j of ``wts[t, j] * y[t * top + j]``; y [T top, d] float32, out [T, d] float32."""
+    _dev(y, "y", torch.float32); _dev(wts, "wts", torch.float32); _dev(out, "out", torch.float32)
+    T, top = wts.shape
+    if y.dim() != 2 or y.shape[0] != T * top or out.shape != (T, y.shape[1]):
+        raise KernelError(f"route_combine: y {tuple(y.shape)}, wts {tuple(wts.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_route_combine(_ptr(y), _ptr(wts), T, top, y.shape[1], _ptr(out), int(bool(accumulate)), _stream()),
+           "route_combine")
 
 
 def sides_norm_add(x, a, b, wa, wb, eps, factor, ssq=None, next_weight=None, xg=None):

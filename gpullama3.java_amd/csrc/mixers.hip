@@ -72,10 +72,15 @@ extern "C" int gl3_concat_rows(const float* a, const float* b, void* out, int ou
 // (or (2j, 2j+1)), by the angle whose cos and sin stand in the run's table [position][rot_dim/2]; `back` turns by
 // minus the angle. With `gate` (rows [T][gate_ld] of the same type, head h's value at column gate_col + h; one run
 // only) every element of head h, rotated or not, is multiplied by sigmoid(gate) afterwards.
+// A run with norm_w (float [head_dim]) is first divided by its root mean square per head (over the head's norm_dim
+// elements, eps inside the root; elements behind them are padding and hold zeros) and multiplied by norm_w.
 struct RotRun {
   int col, heads, head_dim, rot_dim;
   const float* cos_tab;
   const float* sin_tab;
+  const float* norm_w;
+  int norm_dim;
+  float norm_eps;
 };
 
 // With a cache (k_cache not null; three runs: queries, keys, values) the second and third run also go to the token's
@@ -116,32 +121,49 @@ __global__ __launch_bounds__(64) void rotate_heads_kernel(T* __restrict__ rows, 
     p[i] = v;
     if (dst) dst[which == 1 ? gl3_k_offset(in_page, i, r.head_dim) : gl3_v_offset(i, in_page, page_size)] = v;
   };
+  float inv = 1.0f;
+  if (r.norm_w) {      // (the whole head is read before any of it is written: the block is one wave)
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < r.norm_dim; i += 64) {
+      const float v = to_f32<T>(p[i]);
+      ss += v * v;
+    }
+    inv = 1.0f / sqrtf(wave_sum(ss) / (float)r.norm_dim + r.norm_eps);
+  }
+  auto get = [&](int i) {
+    const float v = to_f32<T>(p[i]);
+    return r.norm_w ? v * inv * r.norm_w[i] : v;
+  };
   if (r.cos_tab) {
     for (int j = threadIdx.x; j < half; j += 64) {
       const int i0 = adjacent ? 2 * j : j, i1 = adjacent ? 2 * j + 1 : j + half;
       const float cs = r.cos_tab[(long)pos * half + j];
       const float sn = back ? -r.sin_tab[(long)pos * half + j] : r.sin_tab[(long)pos * half + j];
-      const float v0 = to_f32<T>(p[i0]), v1 = to_f32<T>(p[i1]);
+      const float v0 = get(i0), v1 = get(i1);
       put(i0, from_f32<T>((v0 * cs - v1 * sn) * g));
       put(i1, from_f32<T>((v1 * cs + v0 * sn) * g));
     }
   }
-  if (gate || dst)
-    for (int i = (r.cos_tab ? r.rot_dim : 0) + threadIdx.x; i < r.head_dim; i += 64) put(i, from_f32<T>(to_f32<T>(p[i]) * g));
+  if (gate || dst || r.norm_w)
+    for (int i = (r.cos_tab ? r.rot_dim : 0) + threadIdx.x; i < r.head_dim; i += 64) put(i, from_f32<T>(get(i) * g));
 }
 
 extern "C" int gl3_rotate_heads(void* rows, int dtype, long ld, const int* positions, int n_tokens, const int* cols,
                                 const int* heads, const int* head_dims, const int* rot_dims, const float* const* cos_tabs,
                                 const float* const* sin_tabs, int n_runs, int adjacent, int back, const void* gate,
                                 long gate_ld, int gate_col, void* k_cache, void* v_cache, const int* table_rows,
-                                const int* block_table, int table_stride, int page_size, hipStream_t stream) {
+                                const int* block_table, int table_stride, int page_size, const float* const* norm_ws,
+                                const int* norm_dims, float norm_eps, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(rows && positions && n_tokens > 0 && n_runs >= 1 && n_runs <= 3, "gl3_rotate_heads: bad arguments");
   GL3_REQUIRE(!gate || n_runs == 1, "gl3_rotate_heads: a gate goes with one run of heads");
   RotRun r[3] = {};
   long total = 0;
   for (int i = 0; i < n_runs; ++i) {
-    r[i] = RotRun{cols[i], heads[i], head_dims[i], rot_dims[i], cos_tabs[i], sin_tabs[i]};
+    r[i] = RotRun{cols[i], heads[i], head_dims[i], rot_dims[i], cos_tabs[i], sin_tabs[i], norm_ws ? norm_ws[i] : nullptr,
+                  norm_ws && norm_ws[i] ? norm_dims[i] : 0, norm_eps};
+    GL3_REQUIRE(!r[i].norm_w || (r[i].norm_dim > 0 && r[i].norm_dim <= head_dims[i]),
+                "gl3_rotate_heads: run %d: a norm over %d of %d elements", i, r[i].norm_dim, head_dims[i]);
     GL3_REQUIRE(heads[i] > 0 && head_dims[i] > 0 && rot_dims[i] >= 0 && rot_dims[i] % 2 == 0 && rot_dims[i] <= head_dims[i] &&
                     cols[i] >= 0 && cols[i] + (long)heads[i] * head_dims[i] <= ld && (cos_tabs[i] == nullptr) == (sin_tabs[i] == nullptr),
                 "gl3_rotate_heads: run %d: %d heads of %d (%d rotated) from column %d of rows of %ld", i, heads[i],
@@ -150,8 +172,8 @@ extern "C" int gl3_rotate_heads(void* rows, int dtype, long ld, const int* posit
   }
   GL3_REQUIRE(total <= 65535, "gl3_rotate_heads: %ld heads exceed the grid", total);
   if (k_cache) {
-    GL3_REQUIRE(v_cache && table_rows && block_table && table_stride > 0 && n_runs == 3 && heads[1] == heads[2],
-                "gl3_rotate_heads: a cache write takes queries, keys and values, as many value heads as key heads");
+    GL3_REQUIRE(v_cache && table_rows && block_table && table_stride > 0 && n_runs == 3,
+                "gl3_rotate_heads: a cache write takes queries, keys and values");
     GL3_REQUIRE(page_size > 0 && page_size % 32 == 0 && head_dims[1] % 16 == 0 && head_dims[2] % 16 == 0,
                 "gl3_rotate_heads: the cache lies in tiles: page_size %d must be a multiple of 32, head sizes %d and %d of 16",
                 page_size, head_dims[1], head_dims[2]);
@@ -647,6 +669,43 @@ extern "C" int gl3_head_norm_gate(const float* o, const float* w, const float* g
   if (out_dtype == GL3_F32) head_norm_gate_kernel<float><<<grid, block, 0, stream>>>(o, w, gate, eps, (float*)out, H, D);
   else if (out_dtype == GL3_BF16) head_norm_gate_kernel<bf16_t><<<grid, block, 0, stream>>>(o, w, gate, eps, (bf16_t*)out, H, D);
   else GL3_REQUIRE(false, "gl3_head_norm_gate: unknown dtype %d", out_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- two score maps' outputs into one
+// att [T][ld_a]: head h's output under the first map at column 2 h D, under the second at (2 h + 1) D. out [T][ld_o],
+// head h at h * D: o = a1 - lambda a2, divided by its root mean square over the head's `dim` elements (eps inside
+// the root; elements behind them are padding and hold zeros), times `mult`. One wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void diff_combine_kernel(const T* __restrict__ att, long ld_a, T* __restrict__ out, long ld_o,
+                                                           int H, int D, int dim, float lambda, float eps, float mult) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y;
+  const T* a1 = att + t * ld_a + (long)2 * h * D;
+  const T* a2 = a1 + D;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += 64) {
+    const float o = to_f32<T>(a1[i]) - lambda * to_f32<T>(a2[i]);
+    ss += o * o;
+  }
+  const float f = mult / sqrtf(wave_sum(ss) / (float)dim + eps);
+  T* op = out + t * ld_o + (long)h * D;
+  for (int i = threadIdx.x; i < D; i += 64) op[i] = from_f32<T>((to_f32<T>(a1[i]) - lambda * to_f32<T>(a2[i])) * f);
+}
+
+extern "C" int gl3_diff_combine(const void* att, long ld_a, void* out, long ld_o, int dtype, int n_tokens, int H, int D, int dim,
+                                float lambda, float eps, float mult, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(att && out && n_tokens > 0 && H > 0 && H <= 65535 && D > 0 && dim > 0 && dim <= D && ld_a >= 2L * H * D &&
+                  ld_o >= (long)H * D,
+              "gl3_diff_combine: %d heads of %d (%d used) in rows of %ld and %ld", H, D, dim, ld_a, ld_o);
+  const dim3 grid(n_tokens, H), block(64);
+  if (dtype == GL3_F32)
+    diff_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)att, ld_a, (float*)out, ld_o, H, D, dim, lambda, eps, mult);
+  else if (dtype == GL3_BF16)
+    diff_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)att, ld_a, (bf16_t*)out, ld_o, H, D, dim, lambda, eps, mult);
+  else GL3_REQUIRE(false, "gl3_diff_combine: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;
 }

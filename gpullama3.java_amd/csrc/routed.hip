@@ -1,0 +1,286 @@
+// A mixture of experts: the choice of a token's experts, the rows of (token, choice) pairs ordered by expert, the
+// experts' products over those rows, and the weighted sum per token.
+//
+// A pair's result depends on its token and its expert alone: the order of the pairs inside an expert's run and the
+// tile a pair falls into change nothing, so a token's output does not depend on its batch-mates. Sums over K run in an
+// order that the shapes fix.
+#include "common.h"
+
+#define ROUTE_MAX_TOP 16
+#define ROUTE_MAX_EXPERTS 1024
+
+// ----------------------------------------------------------------- the choice
+// logits [T][E] float. The `top` largest (the lower number wins a tie) -> idx [T][top]; their weights are the softmax
+// over the chosen logits alone -> wts [T][top]. One thread a token.
+__global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ logits, int T, int E, int top,
+                                                         int* __restrict__ idx, float* __restrict__ wts) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (long)t * E;
+  int chosen[ROUTE_MAX_TOP];
+  float val[ROUTE_MAX_TOP];
+  for (int j = 0; j < top; ++j) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
+      const float v = z[e];
+      if (!taken && (best < 0 || v > bv)) {
+        best = e;
+        bv = v;
+      }
+    }
+    chosen[j] = best;
+    val[j] = bv;
+  }
+  float sum = 0.f;
+  const float largest = val[0];          // (the first chosen is the largest)
+  for (int j = 0; j < top; ++j) {
+    val[j] = expf(val[j] - largest);
+    sum += val[j];
+  }
+  for (int j = 0; j < top; ++j) {
+    idx[(long)t * top + j] = chosen[j];
+    wts[(long)t * top + j] = val[j] / sum;
+  }
+}
+
+// ----------------------------------------------------------------- pairs ordered by expert
+// idx [n_pairs] -> offsets [E + 1] (the first place of each expert's run) and sorted [n_pairs] (the pairs, expert by
+// expert). One block.
+__global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict__ idx, int n_pairs, int E,
+                                                           int* __restrict__ offsets, int* __restrict__ sorted) {
+  __shared__ int count[ROUTE_MAX_EXPERTS + 1];
+  __shared__ int cursor[ROUTE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[idx[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = count[e];
+      count[e] = run;
+      cursor[e] = run;
+      run += c;
+    }
+    count[E] = run;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = count[e];
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) sorted[atomicAdd(&cursor[idx[i]], 1)] = i;
+}
+
+extern "C" int gl3_route(const float* logits, int n_tokens, int E, int top, int* idx, float* wts, int* offsets, int* sorted,
+                         hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(logits && idx && wts && offsets && sorted, "gl3_route: null argument");
+  GL3_REQUIRE(n_tokens > 0 && E >= 1 && E <= ROUTE_MAX_EXPERTS && top >= 1 && top <= ROUTE_MAX_TOP && top <= E,
+              "gl3_route: the %d largest of %d experts (at most %d of %d)", top, E, ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS);
+  route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts);
+  GL3_LAUNCH_CHECK();
+  route_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(idx, n_tokens * top, E, offsets, sorted);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- the experts' products
+// out[pair][n] = act(sum_k A[pair / a_div][k] * W[e][n][k]) for every pair of expert e's run. offsets null: one expert
+// over all n_rows rows in their own order (the expert that every token passes). Tiles of TM rows of a run x TN columns;
+// a block finds its run by walking the offsets (at most n_rows / TM + E tiles exist; a block beyond them leaves).
+__device__ __forceinline__ float gl3_expert_act(float v, int act) {
+  if (act == 1) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));        // gelu, the erf form
+  if (act == 2) return gl3_activation<false>(v, GL3_ACT_GELU_TANH);
+  if (act == 3) return gl3_activation<false>(v, GL3_ACT_SILU);
+  return v;
+}
+
+__device__ __forceinline__ bool expert_tile(const int* offsets, int E, int n_rows, int TM, int tile, int* e_out, int* lo_out,
+                                            int* hi_out) {
+  if (!offsets) {
+    *e_out = 0;
+    *lo_out = tile * TM;
+    *hi_out = n_rows;
+    return tile * TM < n_rows;
+  }
+  for (int e = 0; e < E; ++e) {
+    const int lo = offsets[e], hi = offsets[e + 1];
+    const int nt = (hi - lo + TM - 1) / TM;
+    if (tile < nt) {
+      *e_out = e;
+      *lo_out = lo + tile * TM;
+      *hi_out = hi;
+      return true;
+    }
+    tile -= nt;
+  }
+  return false;
+}
+
+#define EG_TM 16
+#define EG_TN 64
+#define EG_TK 32
+template <typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(256) void expert_gemm_generic_kernel(const TA* __restrict__ A, long lda, int a_div,
+                                                                   const TW* __restrict__ W, int N, int K,
+                                                                   const int* __restrict__ offsets,
+                                                                   const int* __restrict__ sorted, int E, int n_rows,
+                                                                   TO* __restrict__ out, long ldo, int act) {
+  __shared__ float sa[EG_TM][EG_TK + 1];
+  __shared__ float sw[EG_TN][EG_TK + 1];
+  __shared__ int rows[EG_TM];
+  int e, lo, hi;
+  if (!expert_tile(offsets, E, n_rows, EG_TM, blockIdx.x, &e, &lo, &hi)) return;
+  const int m = hi - lo < EG_TM ? hi - lo : EG_TM;
+  if (threadIdx.x < EG_TM) rows[threadIdx.x] = threadIdx.x < m ? (sorted ? sorted[lo + threadIdx.x] : lo + threadIdx.x) : -1;
+  __syncthreads();
+  const int n0 = blockIdx.y * EG_TN;
+  const TW* We = W + (long)e * N * K;
+  const int r = threadIdx.x / 16, cg = threadIdx.x % 16;      // this thread: row r, columns cg + 16 j
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += EG_TK) {
+    for (int i = threadIdx.x; i < EG_TM * EG_TK; i += 256) {
+      const int rr = i / EG_TK, kk = i % EG_TK;
+      sa[rr][kk] = (rows[rr] >= 0 && k0 + kk < K) ? to_f32<TA>(A[(long)(rows[rr] / a_div) * lda + k0 + kk]) : 0.f;
+    }
+    for (int i = threadIdx.x; i < EG_TN * EG_TK; i += 256) {
+      const int nn = i / EG_TK, kk = i % EG_TK;
+      sw[nn][kk] = (n0 + nn < N && k0 + kk < K) ? to_f32<TW>(We[(long)(n0 + nn) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < EG_TK; ++kk) {
+      const float a = sa[r][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = fmaf(a, sw[cg + 16 * j][kk], acc[j]);
+    }
+    __syncthreads();
+  }
+  if (rows[r] < 0) return;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + cg + 16 * j;
+    if (n < N) out[(long)rows[r] * ldo + n] = from_f32<TO>(gl3_expert_act(acc[j], act));
+  }
+}
+
+// The same on the matrix cores for bfloat16: a block of 4 waves works a tile of 64 rows x 64 columns, wave w the
+// columns 16 w .. 16 w + 15 of all four row groups; operands come straight from memory, 4 consecutive k a lane (a
+// row of A or of W per lane, as v_mfma_f32_16x16x16_bf16 takes them). K must be a multiple of 16.
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short short4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float float4_t;
+#define EM_TM 64
+#define EM_TN 64
+template <typename TO>
+__global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, long lda, int a_div,
+                                                                const bf16_t* __restrict__ W, int N, int K,
+                                                                const int* __restrict__ offsets,
+                                                                const int* __restrict__ sorted, int E, int n_rows,
+                                                                TO* __restrict__ out, long ldo, int act) {
+  __shared__ int rows[EM_TM];
+  int e, lo, hi;
+  if (!expert_tile(offsets, E, n_rows, EM_TM, blockIdx.x, &e, &lo, &hi)) return;
+  const int m = hi - lo < EM_TM ? hi - lo : EM_TM;
+  if (threadIdx.x < EM_TM) rows[threadIdx.x] = threadIdx.x < m ? (sorted ? sorted[lo + threadIdx.x] : lo + threadIdx.x) : -1;
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int li = lane & 15, kb = (lane >> 4) * 4;           // operand row / column of this lane, and its 4 k
+  const int n = blockIdx.y * EM_TN + wave * 16 + li;
+  const bf16_t* wp = W + ((long)e * N + (n < N ? n : 0)) * K + kb;
+  const bf16_t* ap[4];
+  bool a_ok[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int row = rows[g * 16 + li];
+    a_ok[g] = row >= 0;
+    ap[g] = A + (long)(row >= 0 ? row / a_div : 0) * lda + kb;
+  }
+  float4_t acc[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) acc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+  const int groups = (m + 15) / 16;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    short4_t b = {0, 0, 0, 0};
+    if (n < N) b = *reinterpret_cast<const short4_t*>(wp + k0);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if (g < groups) {
+        short4_t a = {0, 0, 0, 0};
+        if (a_ok[g]) a = *reinterpret_cast<const short4_t*>(ap[g] + k0);
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, acc[g], 0, 0, 0);
+      }
+    }
+  }
+  // a lane holds column li of rows 4 (lane / 16) .. + 3 of every group
+  const int nc = blockIdx.y * EM_TN + wave * 16 + li;
+  if (nc >= N) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = rows[g * 16 + (lane >> 4) * 4 + i];
+      if (row >= 0) out[(long)row * ldo + nc] = from_f32<TO>(gl3_expert_act(acc[g][i], act));
+    }
+  }
+}
+
+extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, const void* W, int w_dtype, int E, int N, int K,
+                               const int* offsets, const int* sorted, int n_rows, void* out, int out_dtype, long ldo, int act,
+                               int use_mfma, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(A && W && out && n_rows > 0 && E >= 1 && N > 0 && K > 0 && a_div >= 1 && lda >= K && ldo >= N,
+              "gl3_expert_gemm: bad arguments");
+  GL3_REQUIRE((offsets == nullptr) == (sorted == nullptr) && (offsets || E == 1),
+              "gl3_expert_gemm: runs and their pairs come together; without them one expert takes every row");
+  GL3_REQUIRE(act >= 0 && act <= 3, "gl3_expert_gemm: unknown activation %d", act);
+  GL3_REQUIRE((N + 63) / 64 <= 65535, "gl3_expert_gemm: %d columns exceed the grid", N);
+  if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 16 == 0 && lda % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(A) % 8 == 0) && (reinterpret_cast<uintptr_t>(W) % 8 == 0)) {
+    const dim3 grid((n_rows + EM_TM - 1) / EM_TM + (offsets ? E : 0), (N + EM_TN - 1) / EM_TN), block(256);
+    if (out_dtype == GL3_BF16)
+      expert_gemm_mfma_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                  sorted, E, n_rows, (bf16_t*)out, ldo, act);
+    else if (out_dtype == GL3_F32)
+      expert_gemm_mfma_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                 sorted, E, n_rows, (float*)out, ldo, act);
+    else GL3_REQUIRE(false, "gl3_expert_gemm: unknown output dtype %d", out_dtype);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
+  const dim3 grid((n_rows + EG_TM - 1) / EG_TM + (offsets ? E : 0), (N + EG_TN - 1) / EG_TN), block(256);
+#define EG_LAUNCH(TA, TW, TO)                                                                                          \
+  expert_gemm_generic_kernel<TA, TW, TO><<<grid, block, 0, stream>>>((const TA*)A, lda, a_div, (const TW*)W, N, K, offsets, \
+                                                                     sorted, E, n_rows, (TO*)out, ldo, act)
+  if (a_dtype == GL3_F32 && w_dtype == GL3_F32 && out_dtype == GL3_F32) EG_LAUNCH(float, float, float);
+  else if (a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && out_dtype == GL3_BF16) EG_LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && out_dtype == GL3_F32) EG_LAUNCH(bf16_t, bf16_t, float);
+  else GL3_REQUIRE(false, "gl3_expert_gemm: dtypes %d x %d -> %d are not built", a_dtype, w_dtype, out_dtype);
+#undef EG_LAUNCH
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- the weighted sum
+// out[t] (+)= sum_j wts[t][j] * y[t * top + j], j in order. One thread an element.
+__global__ void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ wts, int top, int d,
+                                     float* __restrict__ out, int accumulate, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long t = i / d;
+  const int c = i % d;
+  float s = accumulate ? out[i] : 0.f;
+  for (int j = 0; j < top; ++j) s = fmaf(wts[t * top + j], y[(t * top + j) * d + c], s);
+  out[i] = s;
+}
+
+extern "C" int gl3_route_combine(const float* y, const float* wts, int n_tokens, int top, int d, float* out, int accumulate,
+                                 hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(y && wts && out && n_tokens > 0 && top >= 1 && d > 0, "gl3_route_combine: bad arguments");
+  const long n = (long)n_tokens * d;
+  GL3_REQUIRE((n + 255) / 256 < (1L << 31), "gl3_route_combine: too many elements");
+  route_combine_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(y, wts, top, d, out, accumulate, n);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,288 @@
+// Recurrences with a matrix per head and a scalar decay: the state space's and the retention's.
+//
+//   S <- a S + b k v^T,   o = S^T q          S [N, P] in 32-bit per (sequence, head)
+//
+// a and b are numbers per (token, head) or per head; q and k may be shared by several heads (a group). A selective
+// state space is k = B, q = C, v = x, a = exp(-exp(A_log) dt), b = dt; a retention is a = the head's decay, b = N^-1/2.
+// Around it: the short causal convolution with silu that the state space's x, B and C pass, with the last taps - 1
+// inputs of every sequence kept in its slot; the decays and step sizes; and the read-outs' gate and unit norm.
+// Everything here is 32-bit arithmetic with accurate exp; only the last kernel's output takes the activations' type.
+// Every kernel walks a step's tokens in order from what the slot holds, and no sum depends on what else is in the
+// batch, so any cut of a sequence into steps gives the same numbers.
+#include "common.h"
+
+// ----------------------------------------------------------------- convolution, decays and step sizes
+// proj: [T][ld] float, the convolution's inputs from column col_x on (`channels` of them), dt from column col_dt on
+// (`heads`). state: [slot][state_ld], the held inputs from state_off on as [taps - 1][channels], oldest first.
+// act [T][channels] = silu(conv + bias); ab [T][2 * heads] = (exp(-exp(A_log) dt), dt), dt = softplus(dt + dt_bias).
+// grid (T, blocks of 256 channels + blocks of 256 heads).
+__global__ __launch_bounds__(256) void ssm_prep_kernel(const float* __restrict__ proj, long ld, int col_x, int channels,
+                                                        int col_dt, int heads, const float* __restrict__ conv_w,
+                                                        const float* __restrict__ conv_b, int taps,
+                                                        const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                                                        const float* __restrict__ state, long state_ld, long state_off,
+                                                        const int* __restrict__ cu_seqlens, const int* __restrict__ seq_of_token,
+                                                        const int* __restrict__ slot_ids, float* __restrict__ act,
+                                                        float* __restrict__ ab, int conv_blocks) {
+  const int t = blockIdx.x;
+  if ((int)blockIdx.y >= conv_blocks) {
+    const int h = (blockIdx.y - conv_blocks) * 256 + threadIdx.x;
+    if (h >= heads) return;
+    const float z = proj[(long)t * ld + col_dt + h] + dt_bias[h];
+    const float dt = z > 20.f ? z + log1pf(expf(-z)) : log1pf(expf(z));
+    ab[(long)t * 2 * heads + h] = expf(-expf(A_log[h]) * dt);
+    ab[(long)t * 2 * heads + heads + h] = dt;
+    return;
+  }
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int s = seq_of_token[t];
+  const int first = cu_seqlens[s], i = t - first;
+  const float* held = state + (long)slot_ids[s] * state_ld + state_off;
+  float sum = conv_b ? conv_b[c] : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int li = i - (taps - 1 - j);
+    const float v = li >= 0 ? proj[(long)(first + li) * ld + col_x + c] : held[(long)(taps - 1 + li) * channels + c];
+    sum = fmaf(conv_w[(long)c * taps + j], v, sum);
+  }
+  act[(long)t * channels + c] = sum / (1.0f + expf(-sum));
+}
+
+// The held inputs move on: after a step of n tokens a sequence holds its last taps - 1 inputs. grid (B, blocks of 256 channels)
+#define SSM_MAX_TAPS 16
+__global__ __launch_bounds__(256) void ssm_hold_kernel(const float* __restrict__ proj, long ld, int col_x, int channels, int taps,
+                                                        float* __restrict__ state, long state_ld, long state_off,
+                                                        const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int first = cu_seqlens[s], n = cu_seqlens[s + 1] - first;
+  float* held = state + (long)slot_ids[s] * state_ld + state_off;
+  float keep[SSM_MAX_TAPS];
+#pragma unroll
+  for (int r = 0; r < SSM_MAX_TAPS; ++r) {
+    if (r < taps - 1) {
+      const int li = n - (taps - 1) + r;
+      keep[r] = li >= 0 ? proj[(long)(first + li) * ld + col_x + c] : held[(long)(taps - 1 + li) * channels + c];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < SSM_MAX_TAPS; ++r)
+    if (r < taps - 1) held[(long)r * channels + c] = keep[r];
+}
+
+extern "C" int gl3_ssm_prep(const float* proj, long ld, int n_tokens, int n_seqs, int col_x, int channels, int col_dt, int heads,
+                            const float* conv_w, const float* conv_b, int taps, const float* A_log, const float* dt_bias,
+                            float* state, long state_ld, long state_off, const int* cu_seqlens, const int* seq_of_token,
+                            const int* slot_ids, float* act, float* ab, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(proj && conv_w && A_log && dt_bias && state && cu_seqlens && seq_of_token && slot_ids && act && ab,
+              "gl3_ssm_prep: null argument");
+  GL3_REQUIRE(n_tokens > 0 && n_seqs > 0 && n_seqs <= 65535 && channels > 0 && heads > 0 && taps >= 1 && taps <= SSM_MAX_TAPS,
+              "gl3_ssm_prep: %d tokens, %d sequences, %d channels, %d heads, %d taps (at most %d)", n_tokens, n_seqs, channels,
+              heads, taps, SSM_MAX_TAPS);
+  GL3_REQUIRE(col_x >= 0 && col_x + channels <= ld && col_dt >= 0 && col_dt + heads <= ld &&
+                  state_off >= 0 && state_off + (long)(taps - 1) * channels <= state_ld,
+              "gl3_ssm_prep: columns %d+%d, %d+%d of rows of %ld; state %ld+%ld of %ld", col_x, channels, col_dt, heads, ld,
+              state_off, (long)(taps - 1) * channels, state_ld);
+  const int conv_blocks = (channels + 255) / 256, head_blocks = (heads + 255) / 256;
+  ssm_prep_kernel<<<dim3(n_tokens, conv_blocks + head_blocks), dim3(256), 0, stream>>>(
+      proj, ld, col_x, channels, col_dt, heads, conv_w, conv_b, taps, A_log, dt_bias, state, state_ld, state_off, cu_seqlens,
+      seq_of_token, slot_ids, act, ab, conv_blocks);
+  GL3_LAUNCH_CHECK();
+  if (taps > 1) {
+    ssm_hold_kernel<<<dim3(n_seqs, conv_blocks), dim3(256), 0, stream>>>(proj, ld, col_x, channels, taps, state, state_ld,
+                                                                         state_off, cu_seqlens, slot_ids);
+    GL3_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// ----------------------------------------------------------------- the recurrence
+// One block a (sequence, head, tile of up to 256 value columns). Thread (r, p) keeps rows r * NR .. of column p of S in
+// registers; a round of tokens' q, k, v, a, b is staged through shared memory; every thread adds its rows' part of a
+// read-out, the parts of the R row groups are added in their order. The order of every sum depends on N, P and the
+// launch shape alone (which follow from N and P).
+struct ScanArgs {
+  const float* q; long ld_q; int col_q;       // [T][ld_q], head group g at col_q + g * N
+  const float* k; long ld_k; int col_k;
+  const float* v; long ld_v; int col_v;       // head h at col_v + h * P
+  const float* a_tok; const float* b_tok;     // [T][ld_ab] per token and head, or null
+  long ld_ab;
+  const float* a_head;                        // [H] when a_tok is null
+  float b_const;                              // when b_tok is null
+  float* state; long state_ld; long state_off;   // [slot][state_ld], S of head h at state_off + h * N * P as [N][P]
+  const int* cu_seqlens; const int* slot_ids;
+  float* out; long ld_o;                      // [T][ld_o], head h at h * P
+  int H, heads_per_group, N, P, R, round;
+};
+
+template <int NR>
+__global__ void decay_scan_kernel(ScanArgs A) {
+  extern __shared__ float smem[];
+  const int s = blockIdx.x, h = blockIdx.y, g = h / A.heads_per_group;
+  const int N = A.N, P = A.P, R = A.R, CH = A.round;
+  const int pt = blockDim.x / R;                          // columns of this block's tile
+  const int r = threadIdx.x / pt, pl = threadIdx.x % pt, p = blockIdx.z * pt + pl;
+  const bool live = p < P;
+  float* sq = smem;                       // [CH][N]
+  float* sk = sq + CH * N;                // [CH][N]
+  float* sv = sk + CH * N;                // [CH][pt]
+  float* sa = sv + CH * pt;               // [CH]
+  float* sb = sa + CH;                    // [CH]
+  float* part = sb + CH;                  // [CH][R][pt]
+  const int first = A.cu_seqlens[s], n = A.cu_seqlens[s + 1] - first;
+  float* S = A.state + (long)A.slot_ids[s] * A.state_ld + A.state_off + (long)h * N * P;
+  const int n0 = r * NR;
+  float acc[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) acc[i] = (live && n0 + i < N) ? S[(long)(n0 + i) * P + p] : 0.f;
+  const float a_fixed = A.a_tok ? 0.f : A.a_head[h];
+  for (int base = 0; base < n; base += CH) {
+    const int m = n - base < CH ? n - base : CH;
+    __syncthreads();
+    for (int e = threadIdx.x; e < m * N; e += blockDim.x) {
+      const int j = e / N, i = e % N;
+      const long t = first + base + j;
+      sq[j * N + i] = A.q[t * A.ld_q + A.col_q + g * N + i];
+      sk[j * N + i] = A.k[t * A.ld_k + A.col_k + g * N + i];
+    }
+    for (int e = threadIdx.x; e < m * pt; e += blockDim.x) {
+      const int j = e / pt, i = e % pt, col = blockIdx.z * pt + i;
+      sv[j * pt + i] = col < P ? A.v[(long)(first + base + j) * A.ld_v + A.col_v + h * P + col] : 0.f;
+    }
+    for (int j = threadIdx.x; j < m; j += blockDim.x) {
+      const long t = first + base + j;
+      sa[j] = A.a_tok ? A.a_tok[t * A.ld_ab + h] : a_fixed;
+      sb[j] = A.b_tok ? A.b_tok[t * A.ld_ab + h] : A.b_const;
+    }
+    __syncthreads();
+    for (int j = 0; j < m; ++j) {
+      const float a = sa[j], bv = sb[j] * sv[j * pt + pl];
+      const float* kq = sk + j * N + n0;
+      const float* qq = sq + j * N + n0;
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        if (n0 + i < N) {
+          acc[i] = fmaf(a, acc[i], kq[i] * bv);
+          o = fmaf(acc[i], qq[i], o);
+        }
+      }
+      part[(j * R + r) * pt + pl] = o;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < m * pt; e += blockDim.x) {
+      const int j = e / pt, i = e % pt, col = blockIdx.z * pt + i;
+      float o = 0.f;
+      for (int rr = 0; rr < R; ++rr) o += part[(j * R + rr) * pt + i];
+      if (col < P) A.out[(long)(first + base + j) * A.ld_o + h * P + col] = o;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NR; ++i)
+    if (live && n0 + i < N) S[(long)(n0 + i) * P + p] = acc[i];
+}
+
+extern "C" int gl3_decay_scan(const float* q, long ld_q, int col_q, const float* k, long ld_k, int col_k, const float* v,
+                              long ld_v, int col_v, const float* a_tok, const float* b_tok, long ld_ab, const float* a_head,
+                              float b_const, float* state, long state_ld, long state_off, const int* cu_seqlens,
+                              const int* slot_ids, float* out, long ld_o, int n_seqs, int H, int heads_per_group, int N, int P,
+                              hipStream_t stream) {
+  if (n_seqs == 0) return 0;
+  GL3_REQUIRE(q && k && v && state && cu_seqlens && slot_ids && out && (a_tok || a_head), "gl3_decay_scan: null argument");
+  GL3_REQUIRE(n_seqs > 0 && H > 0 && H <= 65535 && heads_per_group > 0 && H % heads_per_group == 0 && N > 0 && N <= 1024 && P > 0,
+              "gl3_decay_scan: %d sequences, %d heads in groups of %d, keys of %d (at most 1024), values of %d", n_seqs, H,
+              heads_per_group, N, P);
+  const int groups = H / heads_per_group;
+  GL3_REQUIRE(col_q >= 0 && col_q + (long)groups * N <= ld_q && col_k >= 0 && col_k + (long)groups * N <= ld_k && col_v >= 0 &&
+                  col_v + (long)H * P <= ld_v && (long)H * P <= ld_o && (!(a_tok || b_tok) || ld_ab >= H) &&
+                  state_off >= 0 && state_off + (long)H * N * P <= state_ld,
+              "gl3_decay_scan: columns do not fit their rows, or the state its slot");
+  // the tile of columns, the row groups and the rows a thread keeps
+  const int pt = P >= 256 ? 256 : P;
+  int R = 256 / pt;
+  if (R > N) R = N;
+  if (R < 1) R = 1;
+  int nr = (N + R - 1) / R;
+  while (nr > 64) {           // more rows than a thread keeps: more row groups
+    R *= 2;
+    nr = (N + R - 1) / R;
+  }
+  const int NRT = nr <= 8 ? 8 : nr <= 16 ? 16 : nr <= 32 ? 32 : 64;      // the rows a thread keeps: the kernel's template
+  R = (N + NRT - 1) / NRT;
+  GL3_REQUIRE(R * pt <= 1024, "gl3_decay_scan: keys of %d with values of %d need %d threads", N, P, R * pt);
+  int round = 16;
+  auto bytes = [&](int ch) { return (size_t)(ch * (2 * N + pt + 2) + ch * R * pt) * sizeof(float); };
+  while (round > 1 && bytes(round) > 60000) round /= 2;
+  GL3_REQUIRE(bytes(round) <= 64000, "gl3_decay_scan: keys of %d with values of %d do not fit shared memory", N, P);
+  ScanArgs A{q, ld_q, col_q, k, ld_k, col_k, v, ld_v, col_v, a_tok, b_tok, ld_ab, a_head, b_const, state, state_ld, state_off,
+             cu_seqlens, slot_ids, out, ld_o, H, heads_per_group, N, P, R, round};
+  const dim3 grid(n_seqs, H, (P + pt - 1) / pt), block(R * pt);
+  const size_t sh = bytes(round);
+  if (NRT == 8) decay_scan_kernel<8><<<grid, block, sh, stream>>>(A);
+  else if (NRT == 16) decay_scan_kernel<16><<<grid, block, sh, stream>>>(A);
+  else if (NRT == 32) decay_scan_kernel<32><<<grid, block, sh, stream>>>(A);
+  else decay_scan_kernel<64><<<grid, block, sh, stream>>>(A);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- gate and unit norm of the read-outs
+// y = o + skip_d[h] * skip_x (skip_d may be null); gate_first: y <- y * silu(gate) and then y / rms over each group of
+// `gsize` channels; else y / rms and then times silu(gate). Times w[c] where w is given. One block a (token, group).
+// o [T][C]; skip_x [T][ld_x] from col_x; gate [T][ld_g] from col_g; out [T][C] in the activations' type.
+template <typename TO>
+__global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ skip_x,
+                                                               long ld_x, int col_x, const float* __restrict__ skip_d,
+                                                               int head_dim, const float* __restrict__ gate, long ld_g,
+                                                               int col_g, const float* __restrict__ w, float eps,
+                                                               int gate_first, int C, int gsize, TO* __restrict__ out) {
+  __shared__ float scratch[16];
+  const long t = blockIdx.x;
+  const int c0 = blockIdx.y * gsize;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < gsize; i += blockDim.x) {
+    const int c = c0 + i;
+    float y = o[t * C + c];
+    if (skip_d) y = fmaf(skip_d[c / head_dim], skip_x[t * ld_x + col_x + c], y);
+    if (gate_first) {
+      const float g = gate[t * ld_g + col_g + c];
+      y *= g / (1.0f + expf(-g));
+    }
+    ss += y * y;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)gsize + eps);
+  for (int i = threadIdx.x; i < gsize; i += blockDim.x) {
+    const int c = c0 + i;
+    float y = o[t * C + c];
+    if (skip_d) y = fmaf(skip_d[c / head_dim], skip_x[t * ld_x + col_x + c], y);
+    const float g = gate[t * ld_g + col_g + c];
+    const float sg = g / (1.0f + expf(-g));
+    y = gate_first ? y * sg * inv : y * inv * sg;
+    if (w) y *= w[c];
+    out[t * C + c] = from_f32<TO>(y);
+  }
+}
+
+extern "C" int gl3_group_norm_gate(const float* o, const float* skip_x, long ld_x, int col_x, const float* skip_d, int head_dim,
+                                   const float* gate, long ld_g, int col_g, const float* w, float eps, int gate_first,
+                                   int n_tokens, int C, int gsize, void* out, int out_dtype, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(o && gate && out && n_tokens > 0 && C > 0 && gsize > 0 && C % gsize == 0 && C / gsize <= 65535,
+              "gl3_group_norm_gate: %d channels in groups of %d", C, gsize);
+  GL3_REQUIRE(!skip_d || (skip_x && head_dim > 0 && C % head_dim == 0 && col_x >= 0 && col_x + C <= ld_x),
+              "gl3_group_norm_gate: the skipped input's columns");
+  GL3_REQUIRE(col_g >= 0 && col_g + C <= ld_g, "gl3_group_norm_gate: the gate's columns");
+  const int threads = gsize >= 256 ? 256 : ((gsize + 63) / 64) * 64;
+  const dim3 grid(n_tokens, C / gsize), block(threads);
+  if (out_dtype == GL3_F32)
+    group_norm_gate_kernel<float><<<grid, block, 0, stream>>>(o, skip_x, ld_x, col_x, skip_d, head_dim, gate, ld_g, col_g, w, eps,
+                                                              gate_first, C, gsize, (float*)out);
+  else if (out_dtype == GL3_BF16)
+    group_norm_gate_kernel<bf16_t><<<grid, block, 0, stream>>>(o, skip_x, ld_x, col_x, skip_d, head_dim, gate, ld_g, col_g, w, eps,
+                                                               gate_first, C, gsize, (bf16_t*)out);
+  else GL3_REQUIRE(false, "gl3_group_norm_gate: unknown dtype %d", out_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

@@ -15,7 +15,11 @@ are rotated by their own position before they are cached, with every head's outp
 position (``value_position``); a gate per head (``head_gate`` among the names: sigmoid of one more row per head of the
 stacked projection, multiplied into the head's output); a constant factor on the output (``out_mult``). The last three
 run on kernels that take any head sizes: one product, one kernel that turns q, k and v in place, the cache write, the
-attention, one kernel that turns the output back and applies the gate.
+attention, one kernel that turns the output back and applies the gate. On the same path: a norm on queries and keys per
+head in front of the rotation (``qk_norm_eps``, in the kernel that turns them), a chunked mask (``chunk``), differential
+attention (``differential``: two score maps per head over the same values; queries and keys then have twice the heads,
+stored head by head as [map 1, map 2], and the cache keeps twice the key heads beside the value heads), and a mixer
+without keys and values of its own (no ``k`` among its names) that only ever reads another entry's.
 """
 from __future__ import annotations
 
@@ -46,9 +50,19 @@ class GQAAttention:
         self.hs_stored, self.vd_stored = self.hs, self.vd
         self.value_position_spec = getattr(spec, "value_position", None)
         self.gated = "head_gate" in spec.names
-        # (rotated values, a gate per head, and a rotation with values of another size run on the kernels for any sizes)
+        self.diff = getattr(spec, "differential", None)
+        self.maps = 2 if self.diff is not None else 1
+        self.Hq, self.Kq = self.H * self.maps, self.Kh * self.maps      # query and key heads as the kernels count them
+        self.qk_norm_eps = getattr(spec, "qk_norm_eps", None)
+        self.chunk = int(getattr(spec, "chunk", None) or 0) or None
+        self.reads_only = "k" not in spec.names
+        if self.chunk and spec.window:
+            raise ValueError("an attention has a window or a chunked mask, not both")
+        # (rotated values, a gate per head, a rotation with values of another size, a norm on queries and keys, several
+        # score maps and a mixer that only reads run on the kernels for any sizes)
         self.general = bool(self.value_position_spec is not None or self.gated
-                            or (spec.position is not None and self.vd != self.hs))
+                            or (spec.position is not None and self.vd != self.hs) or self.qk_norm_eps is not None
+                            or self.diff is not None or self.reads_only)
         if spec.position is None or self.general:
             # (a rotation touches a head's first elements only: zeros behind them stay zeros)
             self.hs, self.vd = -(-self.hs // 16) * 16, -(-self.vd // 16) * 16
@@ -76,8 +90,16 @@ class GQAAttention:
 
     def tensors(self):
         n, d, hs, vd = self.names, self.d, self.hs_stored, self.vd_stored
-        out = {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
-               n["v"]: TensorSpec((self.Kh * vd, d)), n["o"]: TensorSpec((d, self.H * vd))}
+        out = {n["q"]: TensorSpec((self.Hq * hs, d)), n["o"]: TensorSpec((d, self.H * vd))}
+        if not self.reads_only:
+            out.update({n["k"]: TensorSpec((self.Kq * hs, d)), n["v"]: TensorSpec((self.Kh * vd, d))})
+        if self.qk_norm_eps is not None:
+            out[n["q_norm"]] = TensorSpec((hs,), "vector")
+            if not self.reads_only:
+                out[n["k_norm"]] = TensorSpec((hs,), "vector")
+        if self.diff is not None:
+            for k in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2"):
+                out[n[k]] = TensorSpec((hs,), "vector", 0.0, 0.3)
         if self.biased:
             out.update({n["q_bias"]: TensorSpec((self.H * hs,), "vector", 0.0, 0.1),
                         n["k_bias"]: TensorSpec((self.Kh * hs,), "vector", 0.0, 0.1),
@@ -143,25 +165,40 @@ class GQAAttention:
         n = self.names
         if self.biased or "o_bias" in n:
             raise ValueError("an attention with rotated values or a gate per head is built without biases")
-        parts = [weights[n[k]] for k in ("q", "k", "v")] + ([weights[n["head_gate"]]] if self.gated else [])
+        if self.reads_only and self.gated:
+            raise ValueError("an attention without keys and values of its own is built without a gate per head")
+        kinds = ("q",) if self.reads_only else ("q", "k", "v")
+        parts = [weights[n[k]] for k in kinds] + ([weights[n["head_gate"]]] if self.gated else [])
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         rows = sum(p.shape[0] for p in parts)
         pad = torch.zeros((-(-rows // 16) * 16 - rows, self.d), dtype=dt, device=parts[0].device)
         self.w_qkv = torch.cat([p.to(dt) for p in parts] + [pad], dim=0).contiguous()
         lo = 0
-        for k, p in zip(("q", "k", "v", "head_gate"), parts):      # the stored names stay addressable as views
+        for k, p in zip(kinds + ("head_gate",), parts):      # the stored names stay addressable as views
             weights[n[k]] = self.w_qkv[lo:lo + p.shape[0]]
             lo += p.shape[0]
         without = getattr(self, "without", frozenset())
         ops.for_few_rows(self.w_qkv, without=without)
+        self.w_q_rows = self.w_qkv[:self.Hq * self.hs]       # what an entry that reads another's keys and values multiplies
         self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
+        self.q_norm_w = self.k_norm_w = None
+        if self.qk_norm_eps is not None:      # (padded like the heads; the kernel reads them as float)
+            def padded(w):
+                out = torch.zeros(self.hs, dtype=torch.float32, device=w.device)
+                out[:self.hs_stored] = w.float()
+                return out
+            self.q_norm_w = padded(weights[n["q_norm"]])
+            self.k_norm_w = padded(weights[n["k_norm"]]) if not self.reads_only else None
+        if self.diff is not None:
+            lq1, lk1, lq2, lk2 = (weights[n[k]].float() for k in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2"))
+            self.diff_lambda = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum())) + float(self.diff.offset)
         self._load_scales(weights)
         if self._slopes_host is not None:
             self.slopes = torch.tensor(self._slopes_host, dtype=torch.float64).to(torch.float32).to(self.w_qkv.device)
 
     def kv_need(self):
-        return KVNeed(self.Kh, self.hs, self.window, v_head_dim=None if self.vd == self.hs else self.vd,
-                      keep_first=self.keep_first)
+        return KVNeed(self.Kq, self.hs, self.window, v_head_dim=None if self.vd == self.hs else self.vd,
+                      keep_first=self.keep_first, v_heads=None if self.maps == 1 else self.Kh, chunk=self.chunk)
 
     def state_need(self):
         return None
@@ -181,26 +218,42 @@ class GQAAttention:
             q = self._project_unequal(ctx, h, k_cache, v_cache, table, run)
         att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
         ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
-                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first)
+                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first, chunk=self.chunk)
         ops.linear(att, self.w_o, x, epilogue, ctx, bias=self.b_o, col_scale=self.out_scale)
 
     def _forward_general(self, ctx, h, x, run, epilogue, k_cache, v_cache, table):
-        if not run.writes_kv:
+        writes = run.writes_kv
+        if not writes and (self.value_position is not None or self.gated):
             raise ValueError("an attention with rotated values or a gate per head keeps keys and values of its own")
-        T, H, Kh, hs, vd = h.shape[0], self.H, self.Kh, self.hs, self.vd
-        qn, kn, vn = H * hs, Kh * hs, Kh * vd
-        qkv = ctx.buffer("qkvg", (T, self.w_qkv.shape[0]), self.dtype)
-        ops.linear(h, self.w_qkv, qkv, ops.EPI_STORE, ctx)
+        if writes and self.reads_only:
+            raise ValueError("an attention without keys and values of its own must read another entry's")
+        T, H, Hq, Kq, Kh, hs, vd = h.shape[0], self.H, self.Hq, self.Kq, self.Kh, self.hs, self.vd
+        qn, kn, vn = Hq * hs, Kq * hs, Kh * vd
+        w = self.w_qkv if writes else self.w_q_rows
+        qkv = ctx.buffer("qkvg", (T, w.shape[0]), self.dtype)
+        ops.linear(h, w, qkv, ops.EPI_STORE, ctx)
         pos, vpos = self.position, self.value_position
-        # q, k and v turned in place, k and v into the cache as they come out: one kernel
+        # q, k and v normed and turned in place, k and v into the cache as they come out: one kernel
         qk = (pos.rot_dim, pos.cos, pos.sin) if pos is not None else (0, None, None)
         vr = (vpos.rot_dim, vpos.cos, vpos.sin) if vpos is not None else (0, None, None)
-        K.rotate_heads(qkv, ctx.positions, [(0, H, hs) + qk, (qn, Kh, hs) + qk, (qn + kn, Kh, vd) + vr],
-                       adjacent=bool(pos.adjacent if pos is not None else vpos is not None and vpos.adjacent),
-                       cache=(k_cache, v_cache, ops._table_rows(ctx), table, k_cache.shape[2]))
-        att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
-        ops.attention(ctx, qkv, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
-                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first)
+        normed = self.qk_norm_eps is not None
+        if writes:
+            K.rotate_heads(qkv, ctx.positions, [(0, Hq, hs) + qk, (qn, Kq, hs) + qk, (qn + kn, Kh, vd) + vr],
+                           adjacent=bool(pos.adjacent if pos is not None else vpos is not None and vpos.adjacent),
+                           cache=(k_cache, v_cache, ops._table_rows(ctx), table, k_cache.shape[2]),
+                           norms=[(self.q_norm_w, self.hs_stored), (self.k_norm_w, self.hs_stored), None] if normed else None,
+                           norm_eps=self.qk_norm_eps or 0.0)
+        elif pos is not None or normed:
+            K.rotate_heads(qkv, ctx.positions, [(0, Hq, hs) + qk], adjacent=bool(pos is not None and pos.adjacent),
+                           norms=[(self.q_norm_w, self.hs_stored)] if normed else None, norm_eps=self.qk_norm_eps or 0.0)
+        att = ctx.buffer("attn_out", (T, Hq * vd), self.dtype)
+        ops.attention(ctx, qkv, k_cache, v_cache, table, att, Hq, Kq, hs, self.window, self.scale, v_head_dim=vd,
+                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first, chunk=self.chunk,
+                      n_v_heads=Kh if self.maps > 1 else None)
+        if self.diff is not None:
+            # the two maps' outputs of every head into one: a1 - lambda a2, a unit norm per head, the factor 1 - offset
+            both, att = att, ctx.buffer("attn_maps_joined", (T, H * vd), self.dtype)
+            K.diff_combine(both, att, H, vd, self.vd_stored, self.diff_lambda, self.diff.norm_eps, 1.0 - self.diff.offset)
         if vpos is not None or self.gated:
             # every head's output turned back by the query's position, then times the head's gate
             K.rotate_heads(att, ctx.positions,
@@ -234,8 +287,8 @@ class _PaddedHeads:
 
     def __getitem__(self, name):
         p, n, w = self.part, self.part.names, self.weights[name]
-        heads = {n["q"]: (p.H, p.hs_stored, p.hs), n["k"]: (p.Kh, p.hs_stored, p.hs), n["v"]: (p.Kh, p.vd_stored, p.vd),
-                 n.get("q_bias"): (p.H, p.hs_stored, p.hs), n.get("k_bias"): (p.Kh, p.hs_stored, p.hs),
+        heads = {n["q"]: (p.Hq, p.hs_stored, p.hs), n.get("k"): (p.Kq, p.hs_stored, p.hs), n.get("v"): (p.Kh, p.vd_stored, p.vd),
+                 n.get("q_bias"): (p.Hq, p.hs_stored, p.hs), n.get("k_bias"): (p.Kq, p.hs_stored, p.hs),
                  n.get("v_bias"): (p.Kh, p.vd_stored, p.vd)}
         if name in heads and w.shape[0] == heads[name][0] * heads[name][1]:
             H, d_in, d_out = heads[name]

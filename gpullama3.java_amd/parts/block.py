@@ -5,6 +5,7 @@ stream keeps the sum (J/inference/InferenceCore.java:74, :151, :154, :172).
 """
 from __future__ import annotations
 
+from ..csrc import lib as K
 from . import ops
 from .base import build_part, register_part
 
@@ -85,5 +86,61 @@ class ParallelBlock:
         ctx.next_norm = None
 
 
+class OutNormBlock:
+    """The norms stand behind the sublayers: ``x += norm1(mixer(x)); x += norm2(ffn(x))``. Mixer and feed-forward
+    read the residual rows themselves (in a bfloat16 engine their rounding to bfloat16, which the kernel that last
+    wrote the rows leaves beside them) and write their output to a 32-bit buffer (``epilogue=EPI_STORE``); the norm's
+    kernel adds the normalised output into the rows. The block has no ``first_norm``: the decoder hands it whole
+    rows and folds no norm into a product while it runs."""
+
+    def __init__(self, spec, dtype, device):
+        self.dtype = dtype
+        self.mixer_norm = build_part("norm", spec.mixer_norm, dtype=dtype)
+        self.mixer = build_part("mixer", spec.mixer, dtype=dtype, device=device)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, dtype=dtype) if spec.ffn is not None else None
+        self.ffn = build_part("ffn", spec.ffn, dtype=dtype, device=device) if spec.ffn is not None else None
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and not hasattr(n, "add_into"):
+                raise ValueError(f"a norm behind a sublayer must offer add_into; {type(n).__name__} does not")
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def cache_needs(self):
+        return self.mixer.kv_need(), self.mixer.state_need()
+
+    def _input(self, ctx, x):
+        """What a sublayer reads: the rows themselves in a 32-bit engine, else their copy in the activations' type
+        (left by the norm kernel that last wrote the rows, or made here)."""
+        if self.dtype == x.dtype:
+            return x
+        h = ctx.buffer("rows_as_input", tuple(x.shape), self.dtype)
+        made = getattr(ctx, "rows_as_input", None)
+        if made != x.data_ptr():
+            K.cast_rows(x, h)
+        return h
+
+    def forward(self, ctx, x, run):
+        T, d = x.shape
+        cast = ctx.buffer("rows_as_input", (T, d), self.dtype) if self.dtype != x.dtype else None
+        y = ctx.buffer("sublayer_out", (T, d), x.dtype)
+        self.mixer.forward(ctx, self._input(ctx, x), y, run, epilogue=ops.EPI_STORE)
+        watch = getattr(ctx.engine, "after_sublayer", None)      # a caller that looks at a sublayer's output and at the rows behind it
+        if watch is not None:
+            watch(run.entry, "mixer", y)
+        self.mixer_norm.add_into(ctx, x, y, cast)
+        if watch is not None:
+            watch(run.entry, "mixer_added", x)
+        ctx.rows_as_input = x.data_ptr() if cast is not None else None
+        if self.ffn is not None:
+            self.ffn.forward(ctx, self._input(ctx, x), y, epilogue=ops.EPI_STORE)
+            if watch is not None:
+                watch(run.entry, "ffn", y)
+            self.ffn_norm.add_into(ctx, x, y, cast)
+        # (the next block may be of another kind and change the rows through other kernels: the copy is not kept)
+        ctx.rows_as_input = None
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "outnorm", OutNormBlock)
 register_part("block", "parallel", ParallelBlock)

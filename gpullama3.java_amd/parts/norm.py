@@ -55,4 +55,35 @@ class RMSNorm:
         return out
 
 
+class LayerNorm:
+    """``(x - mean) / sqrt(var + eps) * w + b`` over the model width, statistics in 32-bit whatever the engine's type.
+    As a norm in front of a part it hands out the normalised rows; a block whose norms stand behind its sublayers
+    calls ``add_into`` instead: the residual rows take the norm of a sublayer's output."""
+    graph_safe = True      # kernel launches on the current stream only
+
+    def __init__(self, spec, dtype):
+        self.dim, self.eps, self.dtype = spec.dim, spec.eps, dtype
+        self.name, self.bias_name = spec.names["weight"], spec.names["bias"]
+        self.weight = self.bias = None
+
+    def tensors(self):
+        return {self.name: TensorSpec((self.dim,), "vector"), self.bias_name: TensorSpec((self.dim,), "vector", 0.0, 0.1)}
+
+    def load(self, weights):
+        self.weight = weights[self.name].float().contiguous()
+        self.bias = weights[self.bias_name].float().contiguous()
+
+    def __call__(self, ctx, x, rows=None, name="normed"):
+        n = x.shape[0] if rows is None else rows.numel()
+        out = ctx.buffer(name, (n, self.dim), self.dtype)
+        K.layernorm(x, self.weight, self.bias, out, self.eps, rows)
+        return out
+
+    def add_into(self, ctx, x, y, cast=None):
+        """``x += norm(y)``; ``cast`` (the activations' type) receives the new rows of x."""
+        K.layernorm_add(x, y, self.weight, self.bias, self.eps, cast)
+        ops.residual_written(ctx, x)
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)

@@ -457,15 +457,18 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
 
 
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale, v_head_dim=None,
-              slopes=None, sink=None, keep_first=0):
+              slopes=None, sink=None, keep_first=0, chunk=None, n_v_heads=None):
     """``v_head_dim``: the values' size (None: the keys'); ``slopes``: float32 [H], a bias of -slopes[h] * distance
     on the scores; ``sink``: the score of a key without a value that every query sees (None: none); ``keep_first``:
-    with a window, the sequence's first keys that every later query still sees."""
+    with a window, the sequence's first keys that every later query still sees; ``chunk``: n: a query sees the earlier
+    keys of its own run of n positions only; ``n_v_heads``: value heads where several score maps share them
+    (``lib.attention_generic``)."""
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     disabled = _off(ctx)
     extras = dict(slopes=slopes, sink=sink)
     extras["keep_first"] = int(keep_first or 0) if window else 0
-    if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
+    if (q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim)     # (the matrix-core kernels: values of the keys' size,
+            and not chunk and n_v_heads is None):                                        # a window or none, as many value heads as key heads)
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
             T = q.shape[0]
@@ -486,4 +489,5 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
                                        ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
                                        seq_rows=getattr(ctx, "seq_rows", None), **extras)
     return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
-                               head_dim, page, window, scale, v_head_dim=v_head_dim, **extras)
+                               head_dim, page, window, scale, v_head_dim=v_head_dim, chunk=int(chunk or 0), n_v_heads=n_v_heads,
+                               **extras)

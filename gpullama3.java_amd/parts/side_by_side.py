@@ -2,7 +2,9 @@
 with a weight of its own, and ``weight`` times the sum of the two (1/2: their average) is the mixer's output.
 
 Either side is any registered mixer whose ``forward`` takes ``epilogue=ops.EPI_STORE`` (its output then goes to a
-float32 buffer instead of into the residual rows). Keys and values are the one side's that asks for them; states of
+float32 buffer instead of into the residual rows). A description with ``normalised=False`` asks for the plain sum of
+the two outputs instead (each side carries its own factor as its ``out_mult``): no norms, no weights; the second
+side's output projection then adds to what the first one's wrote. Keys and values are the one side's that asks for them; states of
 both sides share the run-order entry's state area, the left side's first.
 """
 from __future__ import annotations
@@ -41,6 +43,9 @@ class SideBySide:
         self.left = build_part("mixer", spec.left, dtype=dtype, device=device)
         self.right = build_part("mixer", spec.right, dtype=dtype, device=device)
         self.factor = float(spec.weight) * float(getattr(spec, "out_mult", 1.0))
+        self.normalised = bool(getattr(spec, "normalised", True))
+        if not self.normalised and self.factor != 1.0:
+            raise ValueError("two mixers side by side without norms carry their factors themselves (out_mult of each side)")
         self.w_left = self.w_right = None
         needs = [s.state_need() for s in (self.left, self.right)]
         if any(n is not None and n.dtype != torch.float32 for n in needs):
@@ -54,7 +59,8 @@ class SideBySide:
         return bool(getattr(self.left, "graph_safe", False) and getattr(self.right, "graph_safe", False))
 
     def tensors(self):
-        out = {self.names["left_norm"]: TensorSpec((self.d,), "vector"), self.names["right_norm"]: TensorSpec((self.d,), "vector")}
+        out = ({self.names["left_norm"]: TensorSpec((self.d,), "vector"), self.names["right_norm"]: TensorSpec((self.d,), "vector")}
+               if self.normalised else {})
         out.update(self.left.tensors())
         out.update(self.right.tensors())
         return out
@@ -64,8 +70,9 @@ class SideBySide:
             side.without = getattr(self, "without", frozenset())
             side.may_hold_once = getattr(self, "may_hold_once", False)
             side.load(weights)
-        self.w_left = weights[self.names["left_norm"]].float().contiguous()
-        self.w_right = weights[self.names["right_norm"]].float().contiguous()
+        if self.normalised:
+            self.w_left = weights[self.names["left_norm"]].float().contiguous()
+            self.w_right = weights[self.names["right_norm"]].float().contiguous()
 
     def kv_need(self):
         return self.left.kv_need() or self.right.kv_need()
@@ -74,9 +81,29 @@ class SideBySide:
         n = sum(self.state_sizes)
         return StateNeed(n, torch.float32) if n else None
 
-    def forward(self, ctx, h, x, run):
+    def _forward_sum(self, ctx, h, x, run, epilogue):
+        """The plain sum: the left side's output projection writes (or adds into) ``x``, the right side's adds to it.
+        No product leaves its sums in slices meanwhile: ``x`` may be a buffer that no norm adds them up for."""
+        next_norm, ctx.next_norm = ctx.next_norm, None
+        fuse, ctx.fuse = getattr(ctx, "fuse", False), False
+        try:
+            lo = 0
+            for side, size, epi in ((self.left, self.state_sizes[0], epilogue), (self.right, self.state_sizes[1], ops.EPI_ADD)):
+                side.forward(_Shifted(ctx, lo, lo + size) if size else ctx, h, x, run, epilogue=epi)
+                lo += size
+        finally:
+            ctx.fuse, ctx.next_norm = fuse, next_norm
+        ops.residual_written(ctx, x)
+
+    def forward(self, ctx, h, x, run, epilogue=ops.EPI_ADD):
         if isinstance(h, ops.Normed):
             h = h.materialize()
+        if not self.normalised:
+            if epilogue == ops.EPI_ADD:
+                ops.settle_residual(ctx, x)
+            return self._forward_sum(ctx, h, x, run, epilogue)
+        if epilogue != ops.EPI_ADD:
+            raise ValueError("two normalised mixers side by side add into the residual rows")
         T = h.shape[0]
         next_norm, ctx.next_norm = ctx.next_norm, None      # neither side completes the residual rows
         outs, lo = [], 0
