@@ -146,10 +146,12 @@ class RetentionSide:
     def __init__(self, c, prefix, eps):
         self.c, self.p, self.eps = c, prefix, eps
         self.S = np.zeros((c["heads"], c["dim"], c["vdim"]))
+        self.conditioning = np.inf            # the smallest |o| / (|S| |q|) of the last call: how much of a read-out survives its sum
 
     def forward(self, W, h, first):
         c, p = self.c, self.p
         T, H, D, Dv = h.shape[0], c["heads"], c["dim"], c["vdim"]
+        self.conditioning = np.inf
         pos = np.arange(first, first + T)
         rot = c["rot"]
         q = turn(linear(h, W[p + "q"]).reshape(T, H, D), pos, rot["base"], rot["dims"], "half")
@@ -160,6 +162,8 @@ class RetentionSide:
             for hd in range(H):
                 self.S[hd] = c["decay"][hd] * self.S[hd] + np.outer(k[t, hd], v[t, hd])
                 o[t, hd] = self.S[hd].T @ q[t, hd]
+                self.conditioning = min(self.conditioning, np.linalg.norm(o[t, hd])
+                                        / (np.linalg.norm(self.S[hd]) * np.linalg.norm(q[t, hd]) + 1e-300))
         o = rms_unit(o, self.eps).reshape(T, H * Dv) * silu(linear(h, W[p + "g"]))
         return linear(o, W[p + "o"])
 
@@ -222,15 +226,20 @@ def expert(W, prefix, h):
     return linear(gelu_erf(linear(h, W[prefix + "up"])), W[prefix + "down"])
 
 
-def routed_feed_forward(W, prefix, c, h):
+def routed_feed_forward(W, prefix, c, h, margins=None):
     """The ``top`` experts with the largest router logits, weighted with the softmax over the chosen logits alone,
-    plus an expert that every token passes."""
-    out = np.zeros((h.shape[0], np.asarray(W[prefix + "shared.down"]).shape[0])) if c.get("shared") else None
+    plus an expert that every token passes. ``margins`` (a list) receives, per token, how far the last chosen logit
+    lies from the first one left out, in units of the size that a logit of this router has (the root mean squares
+    of h's elements and of the router's rows' lengths multiplied)."""
     logits = linear(h, W[prefix + "router"])
     top = c["router"]["top"]
     rows = []
     for t in range(h.shape[0]):
-        chosen = np.argsort(-logits[t], kind="stable")[:top]
+        order = np.argsort(-logits[t], kind="stable")
+        chosen = order[:top]
+        if margins is not None and top < len(order):
+            size = np.sqrt((h[t] ** 2).mean()) * np.sqrt((np.asarray(W[prefix + "router"], np.float64) ** 2).sum(-1).mean())
+            margins.append((logits[t, order[top - 1]] - logits[t, order[top]]) / (size + 1e-300))
         w = softmax(logits[t, chosen])
         rows.append(sum(w[i] * expert(W, f"{prefix}e{e}.", h[t:t + 1])[0] for i, e in enumerate(chosen)))
     y = np.stack(rows)
@@ -241,10 +250,15 @@ def routed_feed_forward(W, prefix, c, h):
 
 # ----------------------------------------------------------------- the decoder
 class Sequence:
-    def __init__(self, config, W):
+    """``noise``: every layer's input is multiplied by 1 + noise * N(0, 1) per element, as a 16-bit engine's rounding
+    would disturb it: the twin of a sequence that tells how far rounding alone moves its logits."""
+
+    def __init__(self, config, W, noise=0.0, seed=0):
         self.c, self.W = config, {k: np.asarray(v, np.float64) for k, v in W.items()}
+        self.noise, self.rng = noise, np.random.default_rng([seed, 123])
         self.eps = config["norm"]["eps"]
         self.n = 0
+        self.margin = np.inf                  # the closest call of any router in the last feed
         self.mixers = []
         for i, lay in enumerate(config["layers"]):
             p, m = f"l{i}.mix.", lay["mixer"]
@@ -262,12 +276,120 @@ class Sequence:
         """Logits [len(tokens), vocab] and the residual rows after every layer [layers, len(tokens), width]."""
         W, eps = self.W, self.eps
         x = W["embed"][list(tokens)]
-        after = []
+        after, margins = [], []
         for i, (lay, mixer) in enumerate(zip(self.c["layers"], self.mixers)):
             p = f"l{i}."
+            if self.noise:
+                x = x * (1.0 + self.noise * self.rng.standard_normal(x.shape))
             x = x + layer_norm(mixer.forward(W, x, self.n), W[p + "norm1"], W[p + "norm1.b"], eps)
             if lay.get("mlp") is not None:
-                x = x + layer_norm(routed_feed_forward(W, p + "mlp.", lay["mlp"], x), W[p + "norm2"], W[p + "norm2.b"], eps)
+                x = x + layer_norm(routed_feed_forward(W, p + "mlp.", lay["mlp"], x, margins), W[p + "norm2"], W[p + "norm2.b"], eps)
             after.append(x)
         self.n += len(tokens)
+        self.margin = min(margins) if margins else np.inf
+        self.conditioning = min([m.right.conditioning for m in self.mixers if isinstance(m, SideBySide)], default=np.inf)
         return linear(layer_norm(x, W["final.norm"], W["final.norm.b"], eps), W["head"]), np.stack(after)
+
+
+def forward(config, W, tokens):
+    """Logits [len(tokens), vocab] of one sequence fed whole."""
+    return Sequence(config, W).feed(tokens)[0]
+
+
+# ----------------------------------------------------------------- weights for the tests
+def tensor_shapes(cfg):
+    """Stored name -> shape of every tensor a configuration asks for."""
+    d = cfg["width"]
+    out = {"embed": (cfg["vocab"], d), "head": (cfg["vocab"], d), "final.norm": (d,), "final.norm.b": (d,)}
+    for i, lay in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", lay["mixer"]
+        out[p + "norm1"], out[p + "norm1.b"] = (d,), (d,)
+        if lay["type"] == "mamba2":
+            inner = m["heads"] * m["vdim"]
+            ch = inner + 2 * m["groups"] * m["state"]
+            out.update({p + "mix.in": (inner + ch + m["heads"], d), p + "mix.conv": (ch, m["conv"]), p + "mix.conv.b": (ch,),
+                        p + "mix.dt_bias": (m["heads"],), p + "mix.A_log": (m["heads"],), p + "mix.D": (m["heads"],),
+                        p + "mix.norm": (inner,), p + "mix.o": (d, inner)})
+        elif lay["type"] == "parallel":
+            L, R = m["left"], m["right"]
+            q = p + "mix.left."
+            out.update({q + "q": (L["heads"] * L["dim"], d), q + "k": (L["kv_heads"] * L["dim"], d),
+                        q + "v": (L["kv_heads"] * L["vdim"], d), q + "q.norm": (L["dim"],), q + "k.norm": (L["dim"],),
+                        q + "o": (d, L["heads"] * L["vdim"])})
+            r = p + "mix.right."
+            out.update({r + "q": (R["heads"] * R["dim"], d), r + "k": (R["heads"] * R["dim"], d),
+                        r + "v": (R["heads"] * R["vdim"], d), r + "g": (R["heads"] * R["vdim"], d),
+                        r + "o": (d, R["heads"] * R["vdim"])})
+        else:
+            q = p + "mix."
+            out.update({q + "q": (m["heads"] * 2 * m["dim"], d), q + "q.norm": (m["dim"],), q + "o": (d, m["heads"] * m["vdim"])})
+            for k in ("lq1", "lk1", "lq2", "lk2"):
+                out[q + k] = (m["dim"],)
+            if m.get("kv_from") is None:
+                out.update({q + "k": (m["kv_heads"] * 2 * m["dim"], d), q + "v": (m["kv_heads"] * m["vdim"], d),
+                            q + "k.norm": (m["dim"],)})
+        mlp = lay.get("mlp")
+        if mlp is not None:
+            out[p + "norm2"], out[p + "norm2.b"] = (d,), (d,)
+            q = p + "mlp."
+            out[q + "router"] = (mlp["router"]["experts"], d)
+            for e in range(mlp["router"]["experts"]):
+                out[f"{q}e{e}.up"], out[f"{q}e{e}.down"] = (mlp["expert"]["ff"], d), (d, mlp["expert"]["ff"])
+            if mlp.get("shared") is not None:
+                out[q + "shared.up"], out[q + "shared.down"] = (mlp["shared"]["ff"], d), (d, mlp["shared"]["ff"])
+    return out
+
+
+def make_weights(cfg, seed):
+    """float32 weights that bfloat16 holds exactly, sized so that every mechanism moves the logits: matrices
+    N(0, 1.5/sqrt(fan-in)), norm weights around one, biases around zero, step sizes and decays spread widely."""
+    import zlib
+    import torch
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        rng = np.random.default_rng([seed, zlib.crc32(name.encode())])
+        last = name.split(".")[-1]
+        if last in ("norm1", "norm2", "norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif last == "b":
+            a = 0.3 * rng.standard_normal(shape)
+        elif last == "dt_bias":
+            a = rng.uniform(-3.0, 1.0, shape)
+        elif last == "A_log":
+            a = rng.uniform(-2.0, 1.0, shape)
+        elif last == "D":
+            a = 1.0 + 0.3 * rng.standard_normal(shape)
+        elif last == "conv":
+            a = 0.5 * rng.standard_normal(shape)
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            a = 0.25 * rng.standard_normal(shape)
+        else:
+            a = rng.standard_normal(shape) * (1.5 / np.sqrt(shape[-1]))
+        out[name] = torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).float().numpy()
+    return out
+
+
+def tokens_with_clear_choices(cfg, W, seed, n, margin=0.1, noise=2.0 ** -8, bound=0.02, conditioning=0.03):
+    """n token ids drawn from a seed at which a 16-bit engine has no close call to make. No router's choice is one: at
+    every token and layer the last chosen logit and the first one left out lie at least ``margin`` (times a logit's
+    size) apart. No retention's read-out is the small rest of a sum that cancels (the first token's is (q . k) v, and
+    its unit norm keeps nothing of q . k but the sign): |o| is at least ``conditioning`` times |S| |q|. And no other
+    place turns rounding into another result: a twin of the sequence whose layers read inputs disturbed by ``noise``
+    stays within ``bound`` of its logits. A bfloat16 engine then differs from the plain implementation by
+    rounding, not by another expert or sign."""
+    import copy
+    rng = np.random.default_rng([seed, 11])
+    seq, twin, out = Sequence(cfg, W), Sequence(cfg, W, noise=noise, seed=seed), []
+    while len(out) < n:
+        for _ in range(400):
+            t = int(rng.integers(0, cfg["vocab"]))
+            trial, trial_twin = copy.deepcopy(seq), copy.deepcopy(twin)
+            a, b = trial.feed([t])[0][0], trial_twin.feed([t])[0][0]
+            d = (b - b.mean()) - (a - a.mean())
+            if trial.margin >= margin and trial.conditioning >= conditioning and np.sqrt((d * d).mean()) < bound * np.sqrt(((a - a.mean()) ** 2).mean()):
+                break
+        else:
+            raise RuntimeError("no token without a close call found")
+        seq, twin = trial, trial_twin
+        out.append(t)
+    return out
