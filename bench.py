@@ -26,6 +26,11 @@ decode throughput of both and their ratio; the default run and its line are not 
 ``--arch nodupel`` does the same for a Nodupel model (every fourth layer a minGRU, the others an attention with
 rotated values, a gate per head and a window that keeps the first keys beside a time mixing with heads of 64; the
 shape's gated feed-forward in every layer; a hashed table of token pairs beside the embedding; no loop).
+``--arch nolatar`` does the same for a Nolatar model (layers in turns of four: a state space with heads of 64 and a
+state of 128, a chunked attention beside a retention, a differential attention, and one more that reads the third's
+keys and values; layer norms behind the sublayers; in every layer a routed feed-forward of 8 experts of a quarter of
+the shape's feed-forward size, two a token, beside a shared expert of that size: the shape's multiply-adds a token
+in three quarters of its feed-forward, 2.25 times its feed-forward weights).
 """
 import argparse
 import json
@@ -110,8 +115,8 @@ def main():
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
-    ap.add_argument("--arch", default="llama", choices=["llama", "melizen", "nodupel"],
-                    help="melizen, nodupel: a model of that design with the shape's sizes beside Llama layers of equal size "
+    ap.add_argument("--arch", default="llama", choices=["llama", "melizen", "nodupel", "nolatar"],
+                    help="melizen, nodupel, nolatar: a model of that design with the shape's sizes beside Llama layers of equal size "
                          "(a line of its own form)")
     ap.add_argument("--without", default="", help="names of fast paths to switch off for a comparison on the same machine, "
                     "comma-separated (parts/ops.py: tiled, packed, fused, wide, ...); the line then says so in `config`")
@@ -124,7 +129,7 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
 
-    if args.arch in ("melizen", "nodupel"):
+    if args.arch in ("melizen", "nodupel", "nolatar"):
         return other_beside_llama(args)
 
     import numpy as np
@@ -346,6 +351,34 @@ def nodupel_config(shape, layers, window=1024, keep_first=4):
             "layers": [gru if i % 4 == 0 else side for i in range(layers)]}
 
 
+def nolatar_config(shape, layers, chunk=1024):
+    """A Nolatar model with the sizes of a Llama shape, layers in turns of four: a state space (heads of 64 over the
+    model's width, a state of 128, 8 groups), a chunked attention with the shape's heads beside a retention (half as
+    many heads, values of twice the keys' size), a differential attention with half the shape's heads (two score
+    maps each, values of the keys' size), and one more that reads the third's keys and values. Every layer has 8
+    experts of a quarter of the shape's feed-forward size, two a token, and a shared expert of that size."""
+    d, F = shape["hidden_size"], shape["intermediate_size"]
+    H, G, hs = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    base = shape.get("rope_theta", 500000.0)
+    mlp = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": F // 4}, "shared": {"ff": F // 4}}
+    rot = {"base": base, "dims": hs}
+    ssm = {"type": "mamba2", "mlp": mlp,
+           "mixer": {"heads": d // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    left = {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5, "rot": rot, "mask": {"size": chunk}}
+    right = {"heads": H // 2, "dim": hs, "vdim": 2 * hs, "rot": rot, "decay": [1.0 - 2.0 ** (-5 - (i % 8)) for i in range(H // 2)]}
+    side = {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": right, "left_scale": 0.6, "right_scale": 1.1}}
+    diff = {"heads": H // 2, "kv_heads": max(1, G // 2), "dim": hs, "vdim": hs, "scale": hs ** -0.5, "diff": 0.6, "rot": rot}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 3:
+            out.append({"type": "attention", "mlp": mlp, "mixer": {**diff, "kv_from": i - 1}})
+        else:
+            out.append([ssm, side, {"type": "attention", "mlp": mlp, "mixer": diff}][kind])
+    return {"architecture": "Nolatar", "vocab": shape["vocab_size"], "width": d, "norm": {"eps": 1e-5},
+            "max_positions": shape["max_position_embeddings"], "layers": out}
+
+
 def other_beside_llama(args):
     """Prefill of one prompt and decode steps at --batch for a model of another design (--arch) and for Llama layers
     of equal size, one after the other on the same machine."""
@@ -361,7 +394,7 @@ def other_beside_llama(args):
     per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     arch = args.arch
-    make = {"melizen": melizen_config, "nodupel": nodupel_config}[arch]
+    make = {"melizen": melizen_config, "nodupel": nodupel_config, "nolatar": nolatar_config}[arch]
     configs = {arch: g.config_from_dict(make(shape, layers)),
                "llama": g.config_from_dict({**shape, "num_hidden_layers": layers})}
     results = {}

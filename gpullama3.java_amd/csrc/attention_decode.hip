@@ -63,7 +63,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits,
-    const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
+    const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
   constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
@@ -84,7 +84,11 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int j = lane & 15, qd = lane >> 4;
   const int heads_here = min(16, g - hg * 16);
-  const int h0 = c * g + hg * 16;
+  // (several score maps over the same values: key head c is map c % maps of group c / maps, read by that map of the
+  // group's g heads, and goes with value head c / maps)
+  const int h0 = maps > 1 ? ((c / maps) * g + hg * 16) * maps + c % maps : c * g + hg * 16;
+  const int hstep = maps > 1 ? maps : 1;      // from one of the block's query heads to the next
+  const int n_v = n_kv / hstep, cv = c / hstep;
 
   // The token's row of the block table: row seq_of_token[t], or (seq_of_token null) row t of a table that the step
   // made of its own tokens' rows. Then nothing stands between the kernel's start and the page numbers: those of the
@@ -96,7 +100,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   for (int b = 0; b < CB; ++b)
     first_pages[b] = __builtin_amdgcn_readfirstlane(bt[min(page_of((wave + b * NW) * 32), table_stride - 1)]);
   const int kv_len = __builtin_amdgcn_readfirstlane(positions[t]) + 1;
-  const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int lo = mask_chunk > 0 ? (kv_len - 1) - (kv_len - 1) % mask_chunk : (window > 0 && kv_len > window) ? kv_len - window : 0;
   // With a window, the sequence's first keep_first keys stay visible (BIAS kernels only). Their chunks that lie before
   // the window's first chunk are numbered in front of it: chunk_lo .. chunk_w - 1 stand for chunks 0 .. chunk_w - chunk_lo - 1.
   const int chunk_w = lo / 32, chunk_hi = (kv_len + 31) / 32;
@@ -112,9 +116,9 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk)
-    qt[kk] = j < heads_here ? *(const bf16x8*)(q + (long)t * q_stride + (long)(h0 + j) * HS + kk * 32 + 8 * qd) : zero8;
+    qt[kk] = j < heads_here ? *(const bf16x8*)(q + (long)t * q_stride + (long)(h0 + j * hstep) * HS + kk * 32 + 8 * qd) : zero8;
 
-  const float slope = (BIAS && slopes && j < heads_here) ? slopes[h0 + j] : 0.f;
+  const float slope = (BIAS && slopes && j < heads_here) ? slopes[h0 + j * hstep] : 0.f;
   float m_run = -INFINITY, l_run = 0.f;   // l_run: this lane's share of the row sum
   f32x4 o[DT];
 #pragma unroll
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
         }
         // values: lane (dim j of the tile, quarter qd) takes keys 8qd..8qd+7 of the chunk: 512
         // consecutive elements of the tile row of 16 dims (gl3_v_offset)
-        const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128 + lane * 8;
+        const bf16_t* vb = v_cache + (page * n_v + cv) * (long)page_size * HS + (long)(po / 8) * 128 + lane * 8;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vt[b][dt] = *(const bf16x8*)(vb + (long)dt * page_size * 16);
       }
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     f[w] = sm_m[w][j] == -INFINITY ? 0.f : __expf(sm_m[w][j] - M);
     L += f[w] * sm_l[w][j];
   }
-  const int h = h0 + j;
+  const int h = h0 + j * hstep;
   for (int dt = wave; dt < DT; dt += NW) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -323,7 +327,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                                     int table_stride, float* part_o, float* part_ml, long part_floats, void* out,
                                     long out_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
                                     int window, float scale, int n_splits, const float* slopes, int has_sink, float sink,
-                                    int keep_first, hipStream_t stream) {
+                                    int keep_first, int mask_chunk, int maps, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && block_table && out && table_stride > 0,
               "gl3_attention_decode: null argument");
@@ -333,6 +337,9 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   GL3_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "gl3_attention_decode: %d heads over %d kv heads", n_heads,
               n_kv);
   GL3_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "gl3_attention_decode: queries must be 16-byte aligned");
+  GL3_REQUIRE(mask_chunk >= 0 && (mask_chunk == 0 || window == 0), "gl3_attention_decode: a chunked mask has no window");
+  GL3_REQUIRE(maps >= 1 && n_kv % maps == 0 && n_heads % maps == 0, "gl3_attention_decode: %d score maps over %d heads and %d key heads",
+              maps, n_heads, n_kv);
   GL3_REQUIRE(n_splits >= 1 && n_splits <= 256, "gl3_attention_decode: n_splits=%d", n_splits);
   if (n_splits > 1)
     GL3_REQUIRE(part_o && part_ml && part_floats >= (long)n_tokens * n_heads * n_splits * (head_dim + 2),
@@ -353,7 +360,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
 #define AD_ARGS                                                                                                       \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table,    \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, n_heads / n_kv, page_size, page_shift, window,  \
-      scale, n_splits, slopes, has_sink, sink, keep_first
+      scale, n_splits, slopes, has_sink, sink, keep_first, mask_chunk, maps
 #define GO(HS)                                                                                                        \
   do {                                                                                                                \
     constexpr int CB = HS <= 64 ? 4 : HS <= 96 ? 3 : 2;                                                               \

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
   constexpr int KROW = HS + 8;            // a key row in shared memory, in elements
@@ -72,11 +72,17 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
   const int heads_here = min(GH, g - hg * GH);
   const int h0 = c * g + hg * GH;
+  // (several score maps over the same values: query and key heads lie head by head as [map 0, map 1, ...]; key head c is
+  // map c % maps of group c / maps, read by that map of the group's g heads, and goes with value head c / maps)
+  auto head_at = [&](int hh) { return maps > 1 ? ((c / maps) * g + hg * GH + hh) * maps + c % maps : h0 + hh; };
+  const int n_v = n_kv / maps, cv = c / maps;
   // the sequence's row of the table: its number in the batch, or what `seq_rows` says (a table with a row per cache slot)
   const int* bt = block_table + (long)(seq_rows ? __builtin_amdgcn_readfirstlane(seq_rows[b]) : b) * table_stride;
   // the block's range of chunks, and the wave's own inside it
   const int blk_first = before + qb * 64, blk_last = before + min(qb * 64 + 63, q_len - 1);
-  const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
+  // the first key that position p sees: its chunk's first (a chunked mask), the window's, or the sequence's
+  auto low_of = [&](int p) { return mask_chunk > 0 ? p - p % mask_chunk : (window > 0 && p + 1 > window) ? p + 1 - window : 0; };
+  const int blk_lo = low_of(blk_first);
   // With a window, the sequence's first keep_first keys stay visible (BIAS kernels only). Their chunks that lie before
   // the window's first chunk ckw are numbered in front of it: ck0 .. ckw - 1 stand for chunks 0 .. ckw - ck0 - 1.
   const int ckw = blk_lo / 32, ck1 = blk_last / 32;
@@ -88,9 +94,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   const int p_mine = before + qi0 + j;                           // position of this lane's query
   const int p_last = before + min(qi0 + 15, q_len - 1);          // last position of the wave
   const int p_first = before + qi0;
-  const int lo_first = (window > 0 && p_first + 1 > window) ? p_first + 1 - window : 0;
-  const int lo_last = (window > 0 && p_last + 1 > window) ? p_last + 1 - window : 0;
-  const int lo_mine = (window > 0 && p_mine + 1 > window) ? p_mine + 1 - window : 0;
+  const int lo_first = low_of(p_first);
+  const int lo_last = low_of(p_last);
+  const int lo_mine = low_of(p_mine);
   const int ck_first = active ? lo_first / 32 : 1, ck_last = active ? p_last / 32 : 0;
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -100,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
       qt[hh][kk] = (q_ok && hh < heads_here)
-                       ? *(const bf16x8*)(q + (long)(tok0 + qi0 + j) * q_stride + (long)(h0 + hh) * HS + kk * 32 + 8 * qd)
+                       ? *(const bf16x8*)(q + (long)(tok0 + qi0 + j) * q_stride + (long)head_at(hh) * HS + kk * 32 + 8 * qd)
                        : zero8;
 
   float m_run[GH], l_run[GH];
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   }
   float sl[GH];                                 // the heads' slopes over the scale: the scores are scaled afterwards
 #pragma unroll
-  for (int hh = 0; hh < GH; ++hh) sl[hh] = (BIAS && slopes && hh < heads_here) ? slopes[h0 + hh] / scale : 0.f;
+  for (int hh = 0; hh < GH; ++hh) sl[hh] = (BIAS && slopes && hh < heads_here) ? slopes[head_at(hh)] / scale : 0.f;
 
   // cache -> registers -> shared memory, 16 bytes a unit: a chunk's keys are 32 consecutive rows
   // of a page, its values 32 consecutive positions of each of the HS rows of the transposed page.
@@ -133,7 +139,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     // (inside a page both lie in tiles, gl3_k_offset and gl3_v_offset: the chunk's keys are still
     // 32 * HS consecutive elements, its values 512 consecutive elements for every 16 dims)
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128;
+    const bf16_t* vb = v_cache + (page * n_v + cv) * (long)page_size * HS + (long)(po / 8) * 128;
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
@@ -259,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     l += __shfl_xor(l, 32, 64);
     if (!q_ok || hh >= heads_here) continue;
     const float inv = 1.0f / l;
-    bf16_t* op = out + (long)(tok0 + qi0 + j) * out_stride + (long)(h0 + hh) * HS + 4 * qd;
+    bf16_t* op = out + (long)(tok0 + qi0 + j) * out_stride + (long)head_at(hh) * HS + 4 * qd;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       bf16x4 r;
@@ -288,7 +294,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
   constexpr int NT = CK / 32;             // score tiles of a chunk of CK keys
@@ -303,7 +309,9 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int g = n_heads / n_kv;
   const int qb = q_blocks - 1 - blockIdx.z;      // the longest query blocks of all heads and sequences first
   const int b = blockIdx.y;
-  const int head = blockIdx.x, c = head / g;   // one query head to a block
+  const int head = blockIdx.x;                 // one query head to a block
+  const int c = maps > 1 ? ((head / maps) / g) * maps + head % maps : head / g;      // (its key head: map head % maps of its group)
+  const int n_v = n_kv / maps, cv = c / maps;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, h = lane >> 5;
@@ -314,7 +322,9 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   // the sequence's row of the table: its number in the batch, or what `seq_rows` says (a table with a row per cache slot)
   const int* bt = block_table + (long)(seq_rows ? __builtin_amdgcn_readfirstlane(seq_rows[b]) : b) * table_stride;
   const int blk_first = before + qb * QB, blk_last = before + min(qb * QB + QB - 1, q_len - 1);
-  const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
+  // the first key that position p sees: its chunk's first (a chunked mask), the window's, or the sequence's
+  auto low_of = [&](int p) { return mask_chunk > 0 ? p - p % mask_chunk : (window > 0 && p + 1 > window) ? p + 1 - window : 0; };
+  const int blk_lo = low_of(blk_first);
   // (kept first keys: as in the kernel above, their chunks before the window's first chunk are numbered in front of it)
   const int ckw = blk_lo / CK, ck1 = blk_last / CK;
   const int ck0 = ckw - (BIAS ? min((keep_first + CK - 1) / CK, ckw) : 0);
@@ -325,9 +335,9 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int p_mine = before + qi0 + n;
   const int p_last = before + min(qi0 + 31, q_len - 1);
   const int p_first = before + qi0;
-  const int lo_first = (window > 0 && p_first + 1 > window) ? p_first + 1 - window : 0;
-  const int lo_last = (window > 0 && p_last + 1 > window) ? p_last + 1 - window : 0;
-  const int lo_mine = (window > 0 && p_mine + 1 > window) ? p_mine + 1 - window : 0;
+  const int lo_first = low_of(p_first);
+  const int lo_last = low_of(p_last);
+  const int lo_mine = low_of(p_mine);
   const int ck_first = active ? lo_first / CK : 1, ck_last = active ? p_last / CK : 0;
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -356,7 +366,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     // (inside a page both lie in tiles, gl3_k_offset and gl3_v_offset: the chunk's keys are still
     // CK * HS consecutive elements, its values CK * 16 consecutive elements for every 16 dims)
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128;
+    const bf16_t* vb = v_cache + (page * n_v + cv) * (long)page_size * HS + (long)(po / 8) * 128;
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
@@ -528,7 +538,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
                                      const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
                                      int max_q_len, int n_heads, int n_kv, int head_dim, int page_size, int window,
                                      float scale, int wide_from, const float* slopes, int has_sink, float sink,
-                                     int keep_first, hipStream_t stream) {
+                                     int keep_first, int mask_chunk, int maps, hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && cu_seqlens && kv_before && block_table && out,
               "gl3_attention_prefill: null argument");
@@ -538,6 +548,9 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   GL3_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "gl3_attention_prefill: %d heads over %d kv heads",
               n_heads, n_kv);
   GL3_REQUIRE(scale > 0.f, "gl3_attention_prefill: the score scale %g must be positive", (double)scale);
+  GL3_REQUIRE(mask_chunk >= 0 && (mask_chunk == 0 || window == 0), "gl3_attention_prefill: a chunked mask has no window");
+  GL3_REQUIRE(maps >= 1 && n_kv % maps == 0 && n_heads % maps == 0, "gl3_attention_prefill: %d score maps over %d heads and %d key heads",
+              maps, n_heads, n_kv);
   GL3_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0,
               "gl3_attention_prefill: queries must be 16-byte aligned, outputs 8-byte aligned");
   const int g = n_heads / n_kv;
@@ -555,7 +568,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   if (wide) {
 #define PF_ARGS                                                                                                     \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table,     \
-      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink, keep_first
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink, keep_first, mask_chunk, maps
 #define GOW(HS, CK, AH, OCC)                                                                                        \
   do {                                                                                                              \
     if (biased) attention_prefill_wide_kernel<HS, CK, AH, OCC, true><<<grid, block, 0, stream>>>(PF_ARGS);          \

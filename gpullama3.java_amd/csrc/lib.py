@@ -96,13 +96,13 @@ def _declare(lib):
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P, F, F, P, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
-        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, I, F, I, P],
+        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
         "gl3_scatter_i32": [P, L, P, P, I, P],
         "gl3_upload": [P, P, L, P],
         "gl3_stage_decode": [P, I, I, P, P, P, I, P, P],
         "gl3_stage_step": [P, P, P, I, P, P, P, I, P, I, I, P],
         "gl3_graph_launch": [P, P],
-        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P, I, F, I, P],
+        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name, None)
@@ -1402,9 +1402,11 @@ def decode_splits(n_tokens, n_heads, n_kv, kv_len, head_dim=64):
 
 
 def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                     page_size, window, scale, n_splits, part_o=None, part_ml=None, slopes=None, sink=None, keep_first=0):
+                     page_size, window, scale, n_splits, part_o=None, part_ml=None, slopes=None, sink=None, keep_first=0,
+                     chunk=0, n_v_heads=None):
     """``slopes`` (float32 [H]): score - slopes[h] * distance; ``sink``: the score of a key without a value that every
-    query sees (None: none); ``keep_first``: with a window, the sequence's first keys that stay visible. One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
+    query sees (None: none); ``keep_first``: with a window, the sequence's first keys that stay visible; ``chunk`` and
+    ``n_v_heads`` as in ``attention_generic``. One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
     are needed when ``n_splits`` > 1 (contiguous, adjacent is not required). ``seq_of_token`` None: token t's
     pages are row t of ``block_table`` (a table of the step's own, as ``token_facts`` makes it)."""
     _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
@@ -1417,7 +1419,10 @@ def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, 
         raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
     if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
-    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
+    n_v = n_kv if n_v_heads is None else int(n_v_heads)
+    if n_kv % n_v or n_heads % (n_kv // n_v) or (chunk and window):
+        raise KernelError(f"attention: {n_heads} heads, {n_kv} key heads, {n_v} value heads, chunk {chunk}, window {window}")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", None, n_v)
     if (positions.numel() != T or block_table.dim() != 2
             or (seq_of_token.numel() != T if seq_of_token is not None else block_table.shape[0] < T)):
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
@@ -1431,7 +1436,8 @@ def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, 
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
         block_table.shape[1], _ptr(part_o), _ptr(part_ml), floats, _ptr(out), out.stride(0), T, n_heads, n_kv,
         head_dim, page_size, int(window or 0), float(scale), n_splits, _slopes(slopes, n_heads, "attention_decode"),
-        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, _stream()), "attention_decode")
+        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v,
+        _stream()), "attention_decode")
 
 
 # ------------------------------------------------------------------ bfloat16 product for many rows
@@ -1516,9 +1522,10 @@ def attention_prefill_fits(head_dim, n_heads, n_kv, page_size):
 
 
 def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, out, max_q_len, n_heads, n_kv,
-                      head_dim, page_size, window, scale, seq_rows=None, wide_from=0, slopes=None, sink=None, keep_first=0):
+                      head_dim, page_size, window, scale, seq_rows=None, wide_from=0, slopes=None, sink=None, keep_first=0,
+                      chunk=0, n_v_heads=None):
     """``slopes`` (float32 [H]): score - slopes[h] * distance; ``sink``: the score of a key without a value that every
-    query sees (None: none). Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
+    query sees (None: none); ``chunk`` and ``n_v_heads`` as in ``attention_generic``. Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
     of the packed ``q`` belong to which sequence and where they sit in it. ``seq_rows`` [B] (optional)
     names each sequence's row of ``block_table``; without it sequence b reads row b. ``wide_from``: from
     how many tokens of the step's longest sequence on the kernel with 128 queries a block runs
@@ -1533,7 +1540,10 @@ def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, o
         raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
     if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
-    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
+    n_v = n_kv if n_v_heads is None else int(n_v_heads)
+    if n_kv % n_v or n_heads % (n_kv // n_v) or (chunk and window):
+        raise KernelError(f"attention: {n_heads} heads, {n_kv} key heads, {n_v} value heads, chunk {chunk}, window {window}")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", None, n_v)
     if cu_seqlens.numel() != B + 1 or block_table.dim() != 2 or max_q_len < 1:
         raise KernelError("attention: cu_seqlens / kv_before / block_table shapes")
     if seq_rows is not None:
@@ -1546,7 +1556,8 @@ def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, o
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(cu_seqlens), _ptr(kv_before), _ptr(block_table),
         _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim,
         page_size, int(window or 0), float(scale), int(wide_from), _slopes(slopes, n_heads, "attention_prefill"),
-        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, _stream()), "attention_prefill")
+        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v,
+        _stream()), "attention_prefill")
 
 
 # ------------------------------------------------------------------ host to device without tensor objects

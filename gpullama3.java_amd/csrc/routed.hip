@@ -225,6 +225,113 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __r
   }
 }
 
+// For many rows: the tiled product of gemm_mfma.hip over an expert's run. A block of 8 waves works 128 rows of one run
+// x 128 columns, a wave 32 x 64 as two tiles of the 32x32x16 instruction; K advances in steps of 64 through two buffers
+// in shared memory (while a step's products run out of one, the next step's operands go from registers into the other
+// and the step after that travels from memory to registers; one barrier a step; rows padded by 16 bytes against bank
+// conflicts). A's rows are gathered through the run's pairs, and the results go to the pairs' own rows.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+#define ET_BM 128
+#define ET_BN 128
+#define ET_BK 64
+#define ET_LD (ET_BK + 8)
+template <typename TO>
+__global__ __launch_bounds__(512) void expert_gemm_tiled_kernel(const bf16_t* __restrict__ A, long lda, int a_div,
+                                                                 const bf16_t* __restrict__ W, int N, int K,
+                                                                 const int* __restrict__ offsets,
+                                                                 const int* __restrict__ sorted, int E, int n_rows,
+                                                                 TO* __restrict__ out, long ldo, int act) {
+  constexpr int NT = 512, NA = ET_BM * 8 / NT, NWC = ET_BN * 8 / NT;
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][ET_BM][ET_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][ET_BN][ET_LD];
+  __shared__ int rows[ET_BM];
+  int e, lo, hi;
+  if (!expert_tile(offsets, E, n_rows, ET_BM, blockIdx.x, &e, &lo, &hi)) return;
+  const int m = hi - lo < ET_BM ? hi - lo : ET_BM;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  if (tid < ET_BM) rows[tid] = tid < m ? (sorted ? sorted[lo + tid] : lo + tid) : -1;
+  __syncthreads();
+  const int wm = wave / 2, wn = wave % 2;
+  const int lr = lane & 31, lh = lane >> 5;
+  const int n0 = blockIdx.y * ET_BN;
+  const bf16_t* We = W + (long)e * N * K;
+  // every load is unconditional: rows beyond the run read the run's first row, columns beyond N the last one,
+  // and their results are dropped
+  long aoff[NA], woff[NWC];
+  int arow_s[NA], wrow_s[NWC];
+  const int scol = (tid & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    arow_s[i] = (tid + NT * i) >> 3;
+    const int src = rows[arow_s[i]] >= 0 ? rows[arow_s[i]] : rows[0];
+    aoff[i] = (long)(src / a_div) * lda;
+  }
+#pragma unroll
+  for (int i = 0; i < NWC; ++i) {
+    wrow_s[i] = (tid + NT * i) >> 3;
+    woff[i] = (long)min(n0 + wrow_s[i], N - 1) * K;
+  }
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8_t ra[NA], rw[NWC];
+  bool r_ok = false;
+  auto fetch = [&](int k0) {
+    const int kf = min(k0, K - 8);                     // the step after the last one reads the last again
+    r_ok = k0 + scol < K;
+    const int col = min(scol, K - 8 - kf);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) ra[i] = *(const bf16x8_t*)(A + aoff[i] + kf + col);
+#pragma unroll
+    for (int i = 0; i < NWC; ++i) rw[i] = *(const bf16x8_t*)(We + woff[i] + kf + col);
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i) *(bf16x8_t*)&As[buf][arow_s[i]][scol] = r_ok ? ra[i] : zero;
+#pragma unroll
+    for (int i = 0; i < NWC; ++i) *(bf16x8_t*)&Ws[buf][wrow_s[i]][scol] = r_ok ? rw[i] : zero;
+  };
+  f32x16_t acc[2];
+#pragma unroll
+  for (int jn = 0; jn < 2; ++jn)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[jn][v] = 0.f;
+  const int arow = wm * 32 + lr, wrow0 = wn * 64 + lr, wrow1 = wn * 64 + 32 + lr;
+  fetch(0);
+  store(0);
+  fetch(ET_BK);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += ET_BK, buf ^= 1) {
+#pragma unroll
+    for (int kk = 0; kk < ET_BK / 16; ++kk) {
+      const int kc = kk * 16 + lh * 8;
+      const bf16x8_t b0 = *(const bf16x8_t*)&Ws[buf][wrow0][kc];
+      const bf16x8_t b1 = *(const bf16x8_t*)&Ws[buf][wrow1][kc];
+      const bf16x8_t a = *(const bf16x8_t*)&As[buf][arow][kc];
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[1], 0, 0, 0);
+      if (kk == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (k0 + ET_BK < K) store(buf ^ 1);
+        fetch(k0 + 2 * ET_BK);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __syncthreads();
+  }
+  // a lane holds C[row(v)][col]: row(v) = 8 * (v / 4) + 4 * (lane / 32) + v % 4 inside a 32 x 32 tile, col = lane % 32
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = rows[wm * 32 + (v >> 2) * 8 + lh * 4 + (v & 3)];
+    if (row < 0) continue;
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      const int n = n0 + wn * 64 + tn * 32 + lr;
+      if (n < N) out[(long)row * ldo + n] = from_f32<TO>(gl3_expert_act(acc[tn][v], act));
+    }
+  }
+}
+
 extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, const void* W, int w_dtype, int E, int N, int K,
                                const int* offsets, const int* sorted, int n_rows, void* out, int out_dtype, long ldo, int act,
                                int use_mfma, hipStream_t stream) {
@@ -235,6 +342,20 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
               "gl3_expert_gemm: runs and their pairs come together; without them one expert takes every row");
   GL3_REQUIRE(act >= 0 && act <= 3, "gl3_expert_gemm: unknown activation %d", act);
   GL3_REQUIRE((N + 63) / 64 <= 65535, "gl3_expert_gemm: %d columns exceed the grid", N);
+  // many rows (an expert's run fills tiles of 128): the tiled kernel
+  if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 8 == 0 && K >= 8 && lda % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0) &&
+      n_rows >= 64 * (offsets ? E : 1) && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
+    const dim3 grid((n_rows + ET_BM - 1) / ET_BM + (offsets ? E : 0), (N + ET_BN - 1) / ET_BN), block(512);
+    if (out_dtype == GL3_BF16)
+      expert_gemm_tiled_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                   sorted, E, n_rows, (bf16_t*)out, ldo, act);
+    else
+      expert_gemm_tiled_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                  sorted, E, n_rows, (float*)out, ldo, act);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
   if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 16 == 0 && lda % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(A) % 8 == 0) && (reinterpret_cast<uintptr_t>(W) % 8 == 0)) {
     const dim3 grid((n_rows + EM_TM - 1) / EM_TM + (offsets ? E : 0), (N + EM_TN - 1) / EM_TN), block(256);

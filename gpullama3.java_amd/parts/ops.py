@@ -467,12 +467,12 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
     disabled = _off(ctx)
     extras = dict(slopes=slopes, sink=sink)
     extras["keep_first"] = int(keep_first or 0) if window else 0
-    if (q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim)     # (the matrix-core kernels: values of the keys' size,
-            and not chunk and n_v_heads is None):                                        # a window or none, as many value heads as key heads)
+    extras.update(chunk=int(chunk or 0), n_v_heads=n_v_heads)
+    if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
             T = q.shape[0]
-            splits = K.decode_splits(T, n_heads, n_kv, ctx.kv_len_hint, head_dim)
+            splits = K.decode_splits(T, n_heads, n_kv, min(ctx.kv_len_hint, chunk) if chunk else ctx.kv_len_hint, head_dim)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
@@ -489,5 +489,4 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
                                        ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
                                        seq_rows=getattr(ctx, "seq_rows", None), **extras)
     return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
-                               head_dim, page, window, scale, v_head_dim=v_head_dim, chunk=int(chunk or 0), n_v_heads=n_v_heads,
-                               **extras)
+                               head_dim, page, window, scale, v_head_dim=v_head_dim, **extras)

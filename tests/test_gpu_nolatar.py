@@ -118,6 +118,27 @@ def attention_on_gpu(q, k, v, positions, dtype, chunk, scale, maps=1, page=64):
     return host(out).reshape(T, Hq, v.shape[2])
 
 
+def attention_on_matrix_cores(q, k, v, positions, chunk, scale, kernel, maps=1, page=64):
+    """The same from the matrix-core kernels (bfloat16, values of the keys' size): ``kernel`` ("decode", splits): one
+    token a sequence; ("prompt", wide_from): the tokens of one sequence, the first of them at positions[0]."""
+    from gpullama3_java_amd.csrc import lib as K
+    T, Hq, D = q.shape
+    kc, vc, table = paged(k, v, page, "bfloat16")
+    out = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device=DEV)
+    qd = dev(q.reshape(T, Hq * D), torch.bfloat16)
+    n_v = v.shape[1] if maps > 1 else None
+    if kernel[0] == "decode":
+        n = kernel[1]
+        part_o = torch.zeros((T, Hq, n, D), dtype=torch.float32, device=DEV) if n > 1 else None
+        part_ml = torch.zeros((T, Hq, n, 2), dtype=torch.float32, device=DEV) if n > 1 else None
+        K.attention_decode(qd, kc, vc, i32(positions), i32([0] * T), table, out, Hq, k.shape[1], D, page, None, scale, n, part_o,
+                           part_ml, chunk=chunk or 0, n_v_heads=n_v)
+    else:
+        K.attention_prefill(qd, kc, vc, i32([0, T]), i32([positions[0]]), table, out, T, Hq, k.shape[1], D, page, None, scale,
+                            wide_from=kernel[1], chunk=chunk or 0, n_v_heads=n_v)
+    return host(out).reshape(T, Hq, D)
+
+
 def plain_attention_at(q, k, v, positions, chunk, scale):
     return np.concatenate([P.softmax_attention(q[t:t + 1], k[:p + 1], v[:p + 1], p, scale, chunk) for t, p in enumerate(positions)])
 
@@ -148,6 +169,51 @@ def test_chunk_edges_with_a_marked_key(H, G, D, Dv, chunk, dtype):
         np.testing.assert_allclose(got, ref, atol=2e-4 if dtype == "float32" else 0.25, err_msg=f"marked {marked}")
         for t, see in enumerate(sees):      # the marked value dominates exactly where the key is visible
             assert (np.abs(got[t]).mean() > 10.0) == see, (marked, positions[t])
+
+
+@pytest.mark.parametrize("kernel", [("decode", 1), ("decode", 3), ("prompt", 1), ("prompt", 10 ** 6)])
+@pytest.mark.parametrize("H, G, D, chunk", [(8, 1, 64, 37), (4, 2, 32, 64), (2, 2, 96, 9), (3, 1, 128, 200), (4, 4, 64, 100)])
+def test_chunk_edges_on_the_matrix_cores(H, G, D, chunk, kernel):
+    """The marked key at a chunk's first and last position and at a page border, against the plain attention: decode
+    steps (one block and three splits of the keys) at positions right at and around the next chunk's start, and prompt
+    steps (both kernels) whose tokens begin in one chunk, behind cached tokens, and end in the next."""
+    rng = np.random.default_rng([H, D, chunk])
+    S = 330
+    for marked in sorted({0, chunk - 1, chunk, 2 * chunk - 1, 64, (200 // chunk) * chunk} & set(range(S))):
+        q, k = bf16_exact(rng.standard_normal((S, H, D)) * 0.3), bf16_exact(rng.standard_normal((S, G, D)) * 0.3)
+        v = bf16_exact(rng.standard_normal((S, G, D)))
+        k[marked] = 0.0
+        k[marked, :, 0] = 6.0
+        q[:, :, 0] = 6.0
+        v[marked] = 30.0
+        edge = (marked // chunk + 1) * chunk
+        if kernel[0] == "decode":
+            positions = sorted({p for p in (marked, marked + 1, edge - 1, edge, edge + 1, 63, 64, 65, 127, 128, 329) if marked <= p < S}
+                               | {0, 1, max(0, marked - 1)})
+        else:
+            first = max(0, marked - 5)
+            positions = list(range(first, min(S, max(edge + 40, first + 150))))
+        ref = plain_attention_at(q[positions], k, v, positions, chunk, 0.25)
+        got = attention_on_matrix_cores(q[positions], k, v, positions, chunk, 0.25, kernel)
+        np.testing.assert_allclose(got, ref, atol=0.25, err_msg=f"marked {marked}")
+        for t, p in enumerate(positions):
+            assert (np.abs(got[t]).mean() > 10.0) == P.sees(p, marked, chunk), (marked, p)
+
+
+@pytest.mark.parametrize("kernel", [("decode", 1), ("decode", 2), ("prompt", 1), ("prompt", 10 ** 6)])
+@pytest.mark.parametrize("H, G, D", [(4, 2, 64), (4, 1, 32), (3, 3, 96), (20, 1, 64), (2, 1, 128)])
+def test_two_score_maps_on_the_matrix_cores(H, G, D, kernel):
+    rng = np.random.default_rng([H, G, D, 5])
+    S = 200
+    q, k = bf16_exact(rng.standard_normal((S, H, 2, D))), bf16_exact(rng.standard_normal((S, G, 2, D)))
+    k[:, :, 1] *= 4.0
+    v = bf16_exact(rng.standard_normal((S, G, D)) + np.arange(G)[None, :, None] * 3.0)
+    positions = [0, 1, 63, 64, 65, 199] if kernel[0] == "decode" else list(range(30, 200))
+    got = attention_on_matrix_cores(q[positions].reshape(-1, H * 2, D), k.reshape(S, G * 2, D), v, positions, None, 0.2, kernel, maps=2)
+    got = got.reshape(len(positions), H, 2, D)
+    for m in range(2):
+        ref = plain_attention_at(q[positions][:, :, m], k[:, :, m], v, positions, None, 0.2)
+        np.testing.assert_allclose(got[:, :, m], ref, atol=0.05, err_msg=f"map {m}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -348,7 +414,8 @@ def test_router_choice_ties_weights_and_runs():
 
 
 @pytest.mark.parametrize("dtype, mfma", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
-@pytest.mark.parametrize("E, top, T, d, F", [(5, 2, 90, 96, 40), (3, 3, 7, 64, 72), (12, 2, 300, 128, 96), (4, 1, 1, 80, 48), (6, 2, 3, 256, 33)])
+@pytest.mark.parametrize("E, top, T, d, F", [(5, 2, 90, 96, 40), (3, 3, 7, 64, 72), (12, 2, 300, 128, 96), (4, 1, 1, 80, 48), (6, 2, 3, 256, 33),
+                                             (4, 2, 700, 200, 136), (2, 1, 1000, 72, 264)])
 def test_experts_products_over_runs_of_pairs(E, top, T, d, F, dtype, mfma):
     """Runs of unequal lengths, experts that nobody chose, more pairs than a tile holds, one token; each pair's hidden
     row and output against the plain expert of its choice."""
