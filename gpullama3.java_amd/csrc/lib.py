@@ -66,7 +66,7 @@ def _declare(lib):
         "gl3_layernorm_add": [P, P, P, P, I, I, F, P, I, P],
         "gl3_cast_rows": [P, P, I, L, P],
         "gl3_ssm_prep": [P, L, I, I, I, I, I, I, P, P, I, P, P, P, L, L, P, P, P, P, P, P],
-        "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P],
+        "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P, L, I, I, P],
         "gl3_group_norm_gate": [P, P, L, I, P, I, P, L, I, P, F, I, I, I, I, P, I, P],
         "gl3_route": [P, I, I, I, P, P, P, P, P],
         "gl3_expert_gemm": [P, I, L, I, P, I, I, I, I, P, P, I, P, I, L, I, I, P],
@@ -644,12 +644,33 @@ def ssm_prep(proj, col_x, channels, col_dt, heads, conv_w, conv_b, A_log, dt_bia
                                   _stream()), "ssm_prep")
 
 
+SCAN_PIECE_BLOCKS = 1024      # a long step's recurrence is cut until about this many (sequence, piece, head) run side by side
+SCAN_PIECE_LEAST = 32         # tokens: shorter pieces cost more in their start states than they gain
+
+
+def scan_piece_len(max_len, n_seqs, H):
+    """The length of the pieces into which ``decay_scan`` cuts a step whose longest sequence has ``max_len`` tokens, or
+    0 for a step in one piece. It follows from the step's shape alone."""
+    want = max(1, SCAN_PIECE_BLOCKS // max(1, n_seqs * H))
+    piece = max(SCAN_PIECE_LEAST, -(-max_len // want))
+    piece = -(-piece // 16) * 16
+    return piece if max_len > piece else 0
+
+
+def scan_pieces_floats(max_len, n_seqs, H, N, P):
+    """Floats of scratch that ``decay_scan`` needs for such a step (0: none)."""
+    piece = scan_piece_len(max_len, n_seqs, H)
+    return n_seqs * -(-max_len // piece) * H * (N * P + 1) if piece else 0
+
+
 def decay_scan(q, col_q, k, col_k, v, col_v, state, state_off, cu_seqlens, slot_ids, out, H, heads_per_group, N, P,
-               a_tok=None, b_tok=None, a_head=None, b_const=1.0):
+               a_tok=None, b_tok=None, a_head=None, b_const=1.0, pieces=None, max_len=0):
     """Per (sequence, head) ``S <- a S + b k v^T`` and ``o = S^T q`` token by token, S [N, P] float32 in ``state``
     [slots, *] from ``state_off + h N P`` on. q and k: float32 rows whose group g (``heads_per_group`` heads share one)
     starts at column ``col + g N``; v: head h at ``col_v + h P``. a and b: per token and head (``a_tok``, ``b_tok``,
-    columns h of rows of the same stride) or per head (``a_head`` [H]) / one number (``b_const``). ``out`` [T, H P]."""
+    columns h of rows of the same stride) or per head (``a_head`` [H]) / one number (``b_const``). ``out`` [T, H P].
+    With ``pieces`` (float32 scratch of ``scan_pieces_floats`` elements) and ``max_len`` (the longest sequence of the
+    step) a long step runs as pieces side by side, joined through their start states."""
     groups = H // heads_per_group
     _f32_rows(q, "q", col_q + groups * N); _f32_rows(k, "k", col_k + groups * N); _f32_rows(v, "v", col_v + H * P)
     _dev(out, "out", torch.float32)
@@ -670,10 +691,18 @@ def decay_scan(q, col_q, k, col_k, v, col_v, state, state_off, cu_seqlens, slot_
     _state_area(state, state_off, H * N * P, "decay_scan")
     _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
     B = cu_seqlens.numel() - 1
+    piece_len = 0
+    if pieces is not None:
+        _dev(pieces, "pieces", torch.float32)
+        if not pieces.is_contiguous() or max_len < 1 or max_len > T:
+            raise KernelError(f"decay_scan: pieces {tuple(pieces.shape)}, the longest of {T} tokens' sequences has {max_len}")
+        piece_len = scan_piece_len(max_len, B, H)
     _check(library().gl3_decay_scan(_ptr(q), q.stride(0), int(col_q), _ptr(k), k.stride(0), int(col_k), _ptr(v), v.stride(0),
                                     int(col_v), _ptr(a_tok), _ptr(b_tok), ld_ab, _ptr(a_head), float(b_const), _ptr(state),
                                     state.stride(0), int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
-                                    out.stride(0), B, int(H), int(heads_per_group), int(N), int(P), _stream()), "decay_scan")
+                                    out.stride(0), B, int(H), int(heads_per_group), int(N), int(P),
+                                    _ptr(pieces) if piece_len else None, pieces.numel() if piece_len else 0, int(max_len),
+                                    int(piece_len), _stream()), "decay_scan")
 
 
 def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=False, skip=None):

@@ -99,9 +99,18 @@ extern "C" int gl3_ssm_prep(const float* proj, long ld, int n_tokens, int n_seqs
 
 // ----------------------------------------------------------------- the recurrence
 // One block a (sequence, head, tile of up to 256 value columns). Thread (r, p) keeps rows r * NR .. of column p of S in
-// registers; a round of tokens' q, k, v, a, b is staged through shared memory; every thread adds its rows' part of a
+// registers; a round of tokens' q, k, v, a, b is staged through shared memory (rows of q and k padded with zeros to
+// R * NR, so the inner loop has no conditions and reads four floats at a time); every thread adds its rows' part of a
 // read-out, the parts of the R row groups are added in their order. The order of every sum depends on N, P and the
 // launch shape alone (which follow from N and P).
+//
+// A long step is cut into pieces of `piece_len` tokens that run side by side (the recurrence is linear in S):
+//   MODE 1  every piece but a sequence's last runs from S = 0 without read-outs and keeps its end state D_c and the
+//           product A_c of its decays;
+//   join    per sequence, piece after piece: the start state of piece c is kept where D_c was, S <- A_c S + D_c;
+//   MODE 2  every piece runs from its start state with read-outs; a sequence's last piece leaves S in the slot.
+// MODE 0 is a step in one piece, from the slot's state and back into it. How a step is cut follows from the launch
+// (lengths and head count), never from the values, and changes a result by rounding alone.
 struct ScanArgs {
   const float* q; long ld_q; int col_q;       // [T][ld_q], head group g at col_q + g * N
   const float* k; long ld_k; int col_k;
@@ -114,37 +123,48 @@ struct ScanArgs {
   const int* cu_seqlens; const int* slot_ids;
   float* out; long ld_o;                      // [T][ld_o], head h at h * P
   int H, heads_per_group, N, P, R, round;
+  float* piece_state;                         // [sequence][piece][H][N][P]
+  float* piece_decay;                         // [sequence][piece][H]
+  int n_pieces, piece_len;
 };
 
-template <int NR>
+template <int NR, int MODE>
 __global__ void decay_scan_kernel(ScanArgs A) {
-  extern __shared__ float smem[];
-  const int s = blockIdx.x, h = blockIdx.y, g = h / A.heads_per_group;
-  const int N = A.N, P = A.P, R = A.R, CH = A.round;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int s = MODE == 0 ? blockIdx.x : blockIdx.x / A.n_pieces, c = MODE == 0 ? 0 : blockIdx.x % A.n_pieces;
+  const int h = blockIdx.y, g = h / A.heads_per_group;
+  const int N = A.N, P = A.P, R = A.R, CH = A.round, NP = R * NR;
+  const int first = A.cu_seqlens[s], n = A.cu_seqlens[s + 1] - first;
+  const int lo = MODE == 0 ? 0 : c * A.piece_len;
+  const int hi = MODE == 0 ? n : (n < lo + A.piece_len ? n : lo + A.piece_len);
+  if (MODE != 0 && lo >= n) return;
+  if (MODE == 1 && hi == n) return;                       // (a sequence's last piece is run once, with read-outs)
   const int pt = blockDim.x / R;                          // columns of this block's tile
   const int r = threadIdx.x / pt, pl = threadIdx.x % pt, p = blockIdx.z * pt + pl;
   const bool live = p < P;
-  float* sq = smem;                       // [CH][N]
-  float* sk = sq + CH * N;                // [CH][N]
-  float* sv = sk + CH * N;                // [CH][pt]
+  float* sq = smem;                       // [CH][NP]
+  float* sk = sq + CH * NP;               // [CH][NP]
+  float* sv = sk + CH * NP;               // [CH][pt]
   float* sa = sv + CH * pt;               // [CH]
   float* sb = sa + CH;                    // [CH]
   float* part = sb + CH;                  // [CH][R][pt]
-  const int first = A.cu_seqlens[s], n = A.cu_seqlens[s + 1] - first;
   float* S = A.state + (long)A.slot_ids[s] * A.state_ld + A.state_off + (long)h * N * P;
+  float* kept = MODE == 0 ? nullptr : A.piece_state + (((long)s * A.n_pieces + c) * A.H + h) * N * P;
+  const float* from = MODE == 0 ? S : kept;
   const int n0 = r * NR;
   float acc[NR];
 #pragma unroll
-  for (int i = 0; i < NR; ++i) acc[i] = (live && n0 + i < N) ? S[(long)(n0 + i) * P + p] : 0.f;
+  for (int i = 0; i < NR; ++i) acc[i] = (MODE != 1 && live && n0 + i < N) ? from[(long)(n0 + i) * P + p] : 0.f;
   const float a_fixed = A.a_tok ? 0.f : A.a_head[h];
-  for (int base = 0; base < n; base += CH) {
-    const int m = n - base < CH ? n - base : CH;
+  float decays = 1.f;
+  for (int base = lo; base < hi; base += CH) {
+    const int m = hi - base < CH ? hi - base : CH;
     __syncthreads();
-    for (int e = threadIdx.x; e < m * N; e += blockDim.x) {
-      const int j = e / N, i = e % N;
+    for (int e = threadIdx.x; e < m * NP; e += blockDim.x) {
+      const int j = e / NP, i = e % NP;
       const long t = first + base + j;
-      sq[j * N + i] = A.q[t * A.ld_q + A.col_q + g * N + i];
-      sk[j * N + i] = A.k[t * A.ld_k + A.col_k + g * N + i];
+      sk[e] = i < N ? A.k[t * A.ld_k + A.col_k + g * N + i] : 0.f;
+      if (MODE != 1) sq[e] = i < N ? A.q[t * A.ld_q + A.col_q + g * N + i] : 0.f;
     }
     for (int e = threadIdx.x; e < m * pt; e += blockDim.x) {
       const int j = e / pt, i = e % pt, col = blockIdx.z * pt + i;
@@ -158,18 +178,28 @@ __global__ void decay_scan_kernel(ScanArgs A) {
     __syncthreads();
     for (int j = 0; j < m; ++j) {
       const float a = sa[j], bv = sb[j] * sv[j * pt + pl];
-      const float* kq = sk + j * N + n0;
-      const float* qq = sq + j * N + n0;
+      const float4* kq = reinterpret_cast<const float4*>(sk + j * NP + n0);
+      const float4* qq = reinterpret_cast<const float4*>(sq + j * NP + n0);
+      if (MODE == 1) decays *= a;
       float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < NR; ++i) {
-        if (n0 + i < N) {
-          acc[i] = fmaf(a, acc[i], kq[i] * bv);
-          o = fmaf(acc[i], qq[i], o);
+      for (int i = 0; i < NR; i += 4) {
+        const float4 kk = kq[i / 4];
+        acc[i] = fmaf(a, acc[i], kk.x * bv);
+        acc[i + 1] = fmaf(a, acc[i + 1], kk.y * bv);
+        acc[i + 2] = fmaf(a, acc[i + 2], kk.z * bv);
+        acc[i + 3] = fmaf(a, acc[i + 3], kk.w * bv);
+        if (MODE != 1) {
+          const float4 qv = qq[i / 4];
+          o = fmaf(acc[i], qv.x, o);
+          o = fmaf(acc[i + 1], qv.y, o);
+          o = fmaf(acc[i + 2], qv.z, o);
+          o = fmaf(acc[i + 3], qv.w, o);
         }
       }
-      part[(j * R + r) * pt + pl] = o;
+      if (MODE != 1) part[(j * R + r) * pt + pl] = o;
     }
+    if (MODE == 1) continue;
     __syncthreads();
     for (int e = threadIdx.x; e < m * pt; e += blockDim.x) {
       const int j = e / pt, i = e % pt, col = blockIdx.z * pt + i;
@@ -178,16 +208,41 @@ __global__ void decay_scan_kernel(ScanArgs A) {
       if (col < P) A.out[(long)(first + base + j) * A.ld_o + h * P + col] = o;
     }
   }
+  if (MODE == 2 && hi != n) return;
+  float* to = MODE == 1 ? kept : S;
 #pragma unroll
   for (int i = 0; i < NR; ++i)
-    if (live && n0 + i < N) S[(long)(n0 + i) * P + p] = acc[i];
+    if (live && n0 + i < N) to[(long)(n0 + i) * P + p] = acc[i];
+  if (MODE == 1 && threadIdx.x == 0 && blockIdx.z == 0) A.piece_decay[((long)s * A.n_pieces + c) * A.H + h] = decays;
 }
 
+// The pieces' start states, sequence by sequence and piece after piece. grid (sequences, H, blocks of 256 elements of S)
+__global__ __launch_bounds__(256) void decay_join_kernel(ScanArgs A) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const long NP = (long)A.N * A.P, e = (long)blockIdx.z * 256 + threadIdx.x;
+  if (e >= NP) return;
+  const int n = A.cu_seqlens[s + 1] - A.cu_seqlens[s];
+  const int pieces = (n + A.piece_len - 1) / A.piece_len;
+  float S = A.state[(long)A.slot_ids[s] * A.state_ld + A.state_off + (long)h * NP + e];
+  for (int c = 0; c < pieces; ++c) {
+    float* kept = A.piece_state + (((long)s * A.n_pieces + c) * A.H + h) * NP + e;
+    if (c + 1 < pieces) {
+      const float d = *kept;
+      *kept = S;
+      S = fmaf(A.piece_decay[((long)s * A.n_pieces + c) * A.H + h], S, d);
+    } else {
+      *kept = S;
+    }
+  }
+}
+
+// `pieces` (null: every step in one piece): room for n_seqs * n_pieces * H * (N * P + 1) floats; a step is cut when its
+// longest sequence (max_len) gives at least two pieces of piece_len tokens.
 extern "C" int gl3_decay_scan(const float* q, long ld_q, int col_q, const float* k, long ld_k, int col_k, const float* v,
                               long ld_v, int col_v, const float* a_tok, const float* b_tok, long ld_ab, const float* a_head,
                               float b_const, float* state, long state_ld, long state_off, const int* cu_seqlens,
                               const int* slot_ids, float* out, long ld_o, int n_seqs, int H, int heads_per_group, int N, int P,
-                              hipStream_t stream) {
+                              float* pieces, long pieces_floats, int max_len, int piece_len, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   GL3_REQUIRE(q && k && v && state && cu_seqlens && slot_ids && out && (a_tok || a_head), "gl3_decay_scan: null argument");
   GL3_REQUIRE(n_seqs > 0 && H > 0 && H <= 65535 && heads_per_group > 0 && H % heads_per_group == 0 && N > 0 && N <= 1024 && P > 0,
@@ -211,19 +266,43 @@ extern "C" int gl3_decay_scan(const float* q, long ld_q, int col_q, const float*
   const int NRT = nr <= 8 ? 8 : nr <= 16 ? 16 : nr <= 32 ? 32 : 64;      // the rows a thread keeps: the kernel's template
   R = (N + NRT - 1) / NRT;
   GL3_REQUIRE(R * pt <= 1024, "gl3_decay_scan: keys of %d with values of %d need %d threads", N, P, R * pt);
+  const int NP = R * NRT;
   int round = 16;
-  auto bytes = [&](int ch) { return (size_t)(ch * (2 * N + pt + 2) + ch * R * pt) * sizeof(float); };
-  while (round > 1 && bytes(round) > 60000) round /= 2;
+  auto bytes = [&](int ch) { return (size_t)(ch * (2 * NP + pt + 2) + ch * R * pt) * sizeof(float); };
+  while (round > 1 && (bytes(round) > 60000 || (round * pt) % 4)) round /= 2;
   GL3_REQUIRE(bytes(round) <= 64000, "gl3_decay_scan: keys of %d with values of %d do not fit shared memory", N, P);
   ScanArgs A{q, ld_q, col_q, k, ld_k, col_k, v, ld_v, col_v, a_tok, b_tok, ld_ab, a_head, b_const, state, state_ld, state_off,
-             cu_seqlens, slot_ids, out, ld_o, H, heads_per_group, N, P, R, round};
-  const dim3 grid(n_seqs, H, (P + pt - 1) / pt), block(R * pt);
+             cu_seqlens, slot_ids, out, ld_o, H, heads_per_group, N, P, R, round, nullptr, nullptr, 1, 0};
+  const int ptiles = (P + pt - 1) / pt;
+  const dim3 block(R * pt);
   const size_t sh = bytes(round);
-  if (NRT == 8) decay_scan_kernel<8><<<grid, block, sh, stream>>>(A);
-  else if (NRT == 16) decay_scan_kernel<16><<<grid, block, sh, stream>>>(A);
-  else if (NRT == 32) decay_scan_kernel<32><<<grid, block, sh, stream>>>(A);
-  else decay_scan_kernel<64><<<grid, block, sh, stream>>>(A);
+#define SCAN_LAUNCH(MODE, grid)                                                          \
+  do {                                                                                   \
+    if (NRT == 8) decay_scan_kernel<8, MODE><<<grid, block, sh, stream>>>(A);            \
+    else if (NRT == 16) decay_scan_kernel<16, MODE><<<grid, block, sh, stream>>>(A);     \
+    else if (NRT == 32) decay_scan_kernel<32, MODE><<<grid, block, sh, stream>>>(A);     \
+    else decay_scan_kernel<64, MODE><<<grid, block, sh, stream>>>(A);                    \
+    GL3_LAUNCH_CHECK();                                                                  \
+  } while (0)
+  const int n_pieces = (pieces && piece_len > 0) ? (max_len + piece_len - 1) / piece_len : 1;
+  if (n_pieces < 2) {
+    SCAN_LAUNCH(0, dim3(n_seqs, H, ptiles));
+    return 0;
+  }
+  const long rows = (long)n_seqs * n_pieces;
+  GL3_REQUIRE(rows < (1L << 31) && rows * H * ((long)N * P + 1) <= pieces_floats,
+              "gl3_decay_scan: %d sequences in %d pieces of %d heads need %ld floats, %ld given", n_seqs, n_pieces, H,
+              rows * H * ((long)N * P + 1), pieces_floats);
+  A.piece_state = pieces;
+  A.piece_decay = pieces + rows * H * (long)N * P;
+  A.n_pieces = n_pieces;
+  A.piece_len = piece_len;
+  const dim3 grid((unsigned)rows, H, ptiles);
+  SCAN_LAUNCH(1, grid);
+  decay_join_kernel<<<dim3(n_seqs, H, (unsigned)(((long)N * P + 255) / 256)), dim3(256), 0, stream>>>(A);
   GL3_LAUNCH_CHECK();
+  SCAN_LAUNCH(2, grid);
+#undef SCAN_LAUNCH
   return 0;
 }
 

@@ -29,9 +29,10 @@ CHUNK_ROWS = 128
 # "fused": norms, rotation and cache write folded into products; "tiled", "packed": the weights' copies in operand
 # order and the rows handed over in the packed tiles' order; "widefold", "wide916": the kernel of whole lines for
 # the gated product with a folded norm and for products of 9 to 16 rows over a long K; "once": a weight whose
-# readers all take the operands' order kept in that order alone (with any switch set, both orders are kept).
+# readers all take the operands' order kept in that order alone (with any switch set, both orders are kept);
+# "scan_pieces": a long step's decayed-matrix recurrence cut into pieces that run side by side.
 SWITCHES = frozenset({"skinny", "wide", "mfma", "attn_decode", "attn_prefill", "fused", "tiled", "packed", "widefold",
-                      "wide916", "once"})
+                      "wide916", "once", "scan_pieces"})
 _NONE = frozenset()
 
 
@@ -383,6 +384,15 @@ def _linear_wide(a, w, out, epilogue, ctx, bias=None, gate=None, col_scale=None)
     residual_written(ctx, out)
     ctx.pending = (out.data_ptr(), part)
     return True
+
+
+def scan_pieces(ctx, H, N, P):
+    """What ``lib.decay_scan`` takes for a step with long sequences: scratch for the pieces' start states and the
+    longest sequence's length (nothing for short steps, which run in one piece)."""
+    n = K.scan_pieces_floats(ctx.max_q_len, ctx.n_seqs, H, N, P)
+    if not n or "scan_pieces" in _off(ctx):
+        return {}
+    return {"pieces": ctx.buffer("scan_pieces", (n,), torch.float32), "max_len": ctx.max_q_len}
 
 
 def _table_rows(ctx):

@@ -84,7 +84,7 @@ class Retention:
             K.rotate_heads(proj, ctx.positions, [(self.off_q, H, D) + rot, (self.off_k, H, D) + rot], adjacent=pos.adjacent)
         o = ctx.buffer("retention_readout", (T, H * Dv), torch.float32)
         K.decay_scan(proj, self.off_q, proj, self.off_k, proj, self.off_v, ctx.slot_state(run.entry), 0, ctx.cu_seqlens,
-                     ctx.slot_ids, o, H, 1, D, Dv, a_head=self.decay, b_const=float(D) ** -0.5)
+                     ctx.slot_ids, o, H, 1, D, Dv, a_head=self.decay, b_const=float(D) ** -0.5, **ops.scan_pieces(ctx, H, D, Dv))
         y = ctx.buffer("retention_out", (T, H * Dv), self.dtype)
         K.group_norm_gate(o, proj, self.off_g, y, Dv, self.spec.norm_eps)
         ops.linear(y, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)

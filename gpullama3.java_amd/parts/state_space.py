@@ -95,7 +95,7 @@ class StateSpace:
                    state, 0, ctx.cu_seqlens, ctx.seq_of_token, ctx.slot_ids, act, ab)
         o = ctx.buffer("ssm_readout", (T, inner), torch.float32)
         K.decay_scan(act, inner + G * N, act, inner, act, 0, state, self.conv_area, ctx.cu_seqlens, ctx.slot_ids, o,
-                     H, H // G, N, P, a_tok=ab[:, :H], b_tok=ab[:, H:])
+                     H, H // G, N, P, a_tok=ab[:, :H], b_tok=ab[:, H:], **ops.scan_pieces(ctx, H, N, P))
         y = ctx.buffer("ssm_out", (T, inner), self.dtype)
         K.group_norm_gate(o, proj, self.off_z, y, inner // self.norm_groups, self.spec.norm_eps, weight=self.norm_w,
                           gate_first=True, skip=(act, 0, self.D, P))

@@ -331,6 +331,68 @@ def test_decayed_matrix_reads_what_was_written_hundreds_of_tokens_ago():
     assert not host(state)[0].any()
 
 
+@pytest.mark.parametrize("H, G, N, P_, lens", [(2, 1, 24, 40, [700, 33, 1, 515]), (5, 5, 16, 16, [129]), (1, 1, 128, 64, [97, 640]),
+                                               (3, 1, 33, 300, [260, 259])])
+def test_decayed_matrix_of_a_long_step_in_pieces_side_by_side(H, G, N, P_, lens):
+    """With scratch for the pieces' start states a long step runs as pieces side by side: sequences of unequal
+    lengths (one of a single token, one shorter than a piece, some that end inside a piece) from states that are not
+    zero give the read-outs and end states of the token-by-token recurrence, with decays per token (some of them
+    close to zero, so that a piece's product of decays underflows) and per head; other slots stay as they are."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng([H, N, P_, len(lens)])
+    n_slots, off = len(lens) + 2, 8
+    slots = list(rng.permutation(n_slots)[:len(lens)])
+    T = sum(lens)
+    piece = K.scan_piece_len(max(lens), len(lens), H)
+    assert piece and max(lens) > piece and any(n % piece for n in lens)
+    q, k = rng.standard_normal((T, G * N)) * 0.3, rng.standard_normal((T, G * N)) * 0.3
+    v = rng.standard_normal((T, H * P_))
+    a, b = rng.uniform(0.8, 1.0, (T, H)), rng.uniform(0.1, 1.0, (T, H))
+    a[rng.random((T, H)) < 0.02] = 1e-30
+    S0 = rng.standard_normal((n_slots, off + H * N * P_))
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    scratch = torch.full((K.scan_pieces_floats(max(lens), len(lens), H, N, P_),), float("nan"), device=DEV)
+    for per_token in (True, False):
+        a_head = rng.uniform(0.9, 0.999, H)
+        aa, bb = (a, b) if per_token else (np.broadcast_to(a_head, (T, H)), np.full((T, H), 0.4))
+        ref_S, ref_o = S0.copy(), np.zeros((T, H, P_))
+        for s, (lo, hi) in enumerate(zip(cu[:-1], cu[1:])):
+            Sm = ref_S[slots[s], off:].reshape(H, N, P_)
+            ref_o[lo:hi] = scan_reference(q[lo:hi].reshape(-1, G, N), k[lo:hi].reshape(-1, G, N), v[lo:hi].reshape(-1, H, P_),
+                                          aa[lo:hi], bb[lo:hi], Sm, H // G)
+        kw = dict(a_tok=dev(aa), b_tok=dev(bb)) if per_token else dict(a_head=dev(a_head), b_const=0.4)
+        state, out = dev(S0), torch.zeros(T, H * P_, device=DEV)
+        K.decay_scan(dev(q), 0, dev(k), 0, dev(v), 0, state, off, i32(cu), i32(slots), out, H, H // G, N, P_,
+                     pieces=scratch, max_len=max(lens), **kw)
+        scale = max(1.0, np.abs(ref_o).max())
+        np.testing.assert_allclose(host(out).reshape(T, H, P_), ref_o, atol=3e-5 * scale)
+        np.testing.assert_allclose(host(state), ref_S, atol=3e-5 * max(1.0, np.abs(ref_S).max()))
+
+
+def test_a_marked_key_is_read_across_many_pieces():
+    """One token writes a value under a key of its own in the step's second piece; a query in a far later piece reads
+    it back scaled by the product of the decays in between, through the pieces' joined start states."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng(5)
+    T, N, P_ = 1500, 32, 16
+    piece = K.scan_piece_len(T, 1, 1)
+    w, r = piece + 3, T - piece - 7
+    k = rng.standard_normal((T, N)) * 0.05
+    k[:, 0] = 0.0
+    k[w] = 0.0
+    k[w, 0] = 1.0
+    v = rng.standard_normal((T, P_)) * 0.05
+    v[w] = 7.0
+    q = np.zeros((T, N))
+    q[r, 0] = 1.0
+    out, state = torch.zeros(T, P_, device=DEV), torch.zeros(2, N * P_, device=DEV)
+    scratch = torch.zeros(K.scan_pieces_floats(T, 1, 1, N, P_), device=DEV)
+    K.decay_scan(dev(q), 0, dev(k), 0, dev(v), 0, state, 0, i32([0, T]), i32([1]), out, 1, 1, N, P_, a_head=dev([0.999]),
+                 b_const=1.0, pieces=scratch, max_len=T)
+    np.testing.assert_allclose(host(out)[r], 7.0 * 0.999 ** (r - w) * np.ones(P_), rtol=3e-4)
+    assert not host(state)[0].any()
+
+
 @pytest.mark.parametrize("taps", [1, 2, 4, 5])
 def test_short_convolution_across_steps(taps):
     """The last taps - 1 inputs of a sequence are part of its state: a prompt in pieces of 1, 2 and more tokens (fewer
