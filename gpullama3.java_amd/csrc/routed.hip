@@ -12,10 +12,8 @@
 // ----------------------------------------------------------------- the choice
 // logits [T][E] float. The `top` largest (the lower number wins a tie) -> idx [T][top]; their weights are the softmax
 // over the chosen logits alone -> wts [T][top]. One thread a token.
-__global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ logits, int T, int E, int top,
-                                                         int* __restrict__ idx, float* __restrict__ wts) {
-  const int t = blockIdx.x * 64 + threadIdx.x;
-  if (t >= T) return;
+__device__ __forceinline__ void route_choose(const float* __restrict__ logits, int t, int E, int top, int* idx,
+                                             float* __restrict__ wts) {
   const float* z = logits + (long)t * E;
   int chosen[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
@@ -46,11 +44,17 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
   }
 }
 
+__global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ logits, int T, int E, int top,
+                                                         int* __restrict__ idx, float* __restrict__ wts) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t < T) route_choose(logits, t, E, top, idx, wts);
+}
+
 // ----------------------------------------------------------------- pairs ordered by expert
 // idx [n_pairs] -> offsets [E + 1] (the first place of each expert's run) and sorted [n_pairs] (the pairs, expert by
 // expert). One block.
-__global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict__ idx, int n_pairs, int E,
-                                                           int* __restrict__ offsets, int* __restrict__ sorted) {
+__device__ __forceinline__ void route_order(const int* idx, int n_pairs, int E, int* __restrict__ offsets,
+                                            int* __restrict__ sorted) {
   __shared__ int count[ROUTE_MAX_EXPERTS + 1];
   __shared__ int cursor[ROUTE_MAX_EXPERTS];
   for (int e = threadIdx.x; e <= E; e += blockDim.x) count[e] = 0;
@@ -72,12 +76,32 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict_
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) sorted[atomicAdd(&cursor[idx[i]], 1)] = i;
 }
 
+__global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict__ idx, int n_pairs, int E,
+                                                           int* __restrict__ offsets, int* __restrict__ sorted) {
+  route_order(idx, n_pairs, E, offsets, sorted);
+}
+
+// Both in one launch for a step of at most 1024 tokens (a thread a token, then the block orders the pairs).
+__global__ __launch_bounds__(1024) void route_few_kernel(const float* __restrict__ logits, int T, int E, int top,
+                                                          int* idx, float* __restrict__ wts,
+                                                          int* __restrict__ offsets, int* __restrict__ sorted) {
+  if ((int)threadIdx.x < T) route_choose(logits, threadIdx.x, E, top, idx, wts);
+  __threadfence_block();
+  __syncthreads();
+  route_order(idx, T * top, E, offsets, sorted);
+}
+
 extern "C" int gl3_route(const float* logits, int n_tokens, int E, int top, int* idx, float* wts, int* offsets, int* sorted,
                          hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(logits && idx && wts && offsets && sorted, "gl3_route: null argument");
   GL3_REQUIRE(n_tokens > 0 && E >= 1 && E <= ROUTE_MAX_EXPERTS && top >= 1 && top <= ROUTE_MAX_TOP && top <= E,
               "gl3_route: the %d largest of %d experts (at most %d of %d)", top, E, ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS);
+  if (n_tokens <= 64) {
+    route_few_kernel<<<dim3(1), dim3(1024), 0, stream>>>(logits, n_tokens, E, top, idx, wts, offsets, sorted);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
   route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts);
   GL3_LAUNCH_CHECK();
   route_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(idx, n_tokens * top, E, offsets, sorted);
@@ -225,6 +249,68 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __r
   }
 }
 
+// For few rows (decode steps: an expert's run is a handful of pairs, and the time goes into reading its weights
+// once): a block of 8 waves works a tile of 16 rows of one run x 16 columns, wave w a slice of K (the slices follow
+// from K alone), 32 k a step with v_mfma_f32_16x16x32_bf16: a lane holds 8 consecutive k of a row of A and of a row
+// of W, read 16 bytes at a time, four steps in flight. The slices' sums are added in their order through shared memory.
+typedef __bf16 bf16x8_few_t __attribute__((ext_vector_type(8)));
+#define EF_WAVES 8
+#define EF_TM 16
+#define EF_TN 16
+template <typename TO>
+__global__ __launch_bounds__(EF_WAVES * 64) void expert_gemm_few_kernel(const bf16_t* __restrict__ A, long lda, int a_div,
+                                                                        const bf16_t* __restrict__ W, int N, int K,
+                                                                        const int* __restrict__ offsets,
+                                                                        const int* __restrict__ sorted, int E, int n_rows,
+                                                                        TO* __restrict__ out, long ldo, int act) {
+  __shared__ int rows[EF_TM];
+  __shared__ float part[EF_WAVES][EF_TM][EF_TN + 1];
+  int e, lo, hi;
+  if (!expert_tile(offsets, E, n_rows, EF_TM, blockIdx.x, &e, &lo, &hi)) return;
+  const int m = hi - lo < EF_TM ? hi - lo : EF_TM;
+  if (threadIdx.x < EF_TM) rows[threadIdx.x] = threadIdx.x < m ? (sorted ? sorted[lo + threadIdx.x] : lo + threadIdx.x) : -1;
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int li = lane & 15, kg = (lane >> 4) * 8;
+  const int n = blockIdx.y * EF_TN + li;
+  const int per = ((K + 31) / 32 + EF_WAVES - 1) / EF_WAVES * 32;       // this wave's slice of K
+  const int k_lo = wave * per, k_hi = k_lo + per < K ? k_lo + per : K;
+  const int row = rows[li];
+  const bf16_t* wp = W + ((long)e * N + (n < N ? n : N - 1)) * K + kg;
+  const bf16_t* ap = A + (long)(row >= 0 ? row / a_div : rows[0] / a_div) * lda + kg;
+  const bf16x8_few_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  int k0 = k_lo;
+  for (; k0 + 128 <= k_hi; k0 += 128) {
+    bf16x8_few_t a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      b[u] = *reinterpret_cast<const bf16x8_few_t*>(wp + k0 + 32 * u);
+      a[u] = *reinterpret_cast<const bf16x8_few_t*>(ap + k0 + 32 * u);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], acc, 0, 0, 0);
+  }
+  for (; k0 < k_hi; k0 += 32) {
+    const bool in = k0 + kg < k_hi;                     // (K is a multiple of 8: a lane's 8 k lie inside or outside)
+    const bf16x8_few_t b = in ? *reinterpret_cast<const bf16x8_few_t*>(wp + k0) : zero;
+    const bf16x8_few_t a = in ? *reinterpret_cast<const bf16x8_few_t*>(ap + k0) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+  // a lane holds column li of rows 4 (lane / 16) .. + 3
+#pragma unroll
+  for (int i = 0; i < 4; ++i) part[wave][(lane >> 4) * 4 + i][li] = acc[i];
+  __syncthreads();
+  if (threadIdx.x < EF_TM * EF_TN) {
+    const int r = threadIdx.x / EF_TN, c = threadIdx.x % EF_TN;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < EF_WAVES; ++w) sum += part[w][r][c];
+    const int nc = blockIdx.y * EF_TN + c;
+    if (rows[r] >= 0 && nc < N) out[(long)rows[r] * ldo + nc] = from_f32<TO>(gl3_expert_act(sum, act));
+  }
+}
+
 // For many rows: the tiled product of gemm_mfma.hip over an expert's run. A block of 8 waves works 128 rows of one run
 // x 128 columns, a wave 32 x 64 as two tiles of the 32x32x16 instruction; K advances in steps of 64 through two buffers
 // in shared memory (while a step's products run out of one, the next step's operands go from registers into the other
@@ -353,6 +439,20 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
     else
       expert_gemm_tiled_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
                                                                   sorted, E, n_rows, (float*)out, ldo, act);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
+  // few rows (an expert's run is a tile of 16 or two): the kernel that reads each weight row in long pieces, K in slices
+  if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 8 == 0 && lda % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0) &&
+      n_rows <= 32 * (offsets ? E : 1) && (N + EF_TN - 1) / EF_TN <= 65535 && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
+    const dim3 grid((n_rows + EF_TM - 1) / EF_TM + (offsets ? E : 0), (N + EF_TN - 1) / EF_TN), block(EF_WAVES * 64);
+    if (out_dtype == GL3_BF16)
+      expert_gemm_few_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                 sorted, E, n_rows, (bf16_t*)out, ldo, act);
+    else
+      expert_gemm_few_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
+                                                                sorted, E, n_rows, (float*)out, ldo, act);
     GL3_LAUNCH_CHECK();
     return 0;
   }

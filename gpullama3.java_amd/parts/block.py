@@ -91,7 +91,9 @@ class OutNormBlock:
     read the residual rows themselves (in a bfloat16 engine their rounding to bfloat16, which the kernel that last
     wrote the rows leaves beside them) and write their output to a 32-bit buffer (``epilogue=EPI_STORE``); the norm's
     kernel adds the normalised output into the rows. The block has no ``first_norm``: the decoder hands it whole
-    rows and folds no norm into a product while it runs."""
+    rows and folds no norm into a product while it runs. The copy that the last norm kernel left stays valid for the
+    next block of this kind (``keeps_rows_copy``: the decoder forgets it before anything else touches the rows)."""
+    keeps_rows_copy = True
 
     def __init__(self, spec, dtype, device):
         self.dtype = dtype
@@ -137,8 +139,6 @@ class OutNormBlock:
             if watch is not None:
                 watch(run.entry, "ffn", y)
             self.ffn_norm.add_into(ctx, x, y, cast)
-        # (the next block may be of another kind and change the rows through other kernels: the copy is not kept)
-        ctx.rows_as_input = None
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -174,6 +174,7 @@ class DecoderModel:
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
         ctx.ssq = ctx.pending = ctx.next_norm = None   # a context may run more than one forward pass: nothing is left over
         ctx.token_facts, ctx.token_tables = {}, {}
+        ctx.rows_as_input = None        # (the address of rows whose copy in the activations' type a block has left)
         order = [self.blocks[r.layer] for r in self.spec.run_order]
         # the norm that reads the residual rows after entry i of the run order, where the block says which
         firsts = [getattr(b, "first_norm", lambda: None)() for b in order] + [self.final_norm]
@@ -208,6 +209,8 @@ class DecoderModel:
             K.embed(self.embedding, ctx.token_ids, embedded, **around)
         for i, (run, block) in enumerate(zip(self.runs, order)):
             before = getattr(self.spec.run_order[i], "before", None)
+            if before is not None or not getattr(block, "keeps_rows_copy", False):
+                ctx.rows_as_input = None
             if before is not None and hasattr(before, "weight_name"):
                 # x <- W [x; x0]: the rows and the embedding's output side by side as the product's input
                 ops.settle_residual(ctx, x)

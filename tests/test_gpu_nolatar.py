@@ -477,7 +477,8 @@ def test_router_choice_ties_weights_and_runs():
 
 @pytest.mark.parametrize("dtype, mfma", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
 @pytest.mark.parametrize("E, top, T, d, F", [(5, 2, 90, 96, 40), (3, 3, 7, 64, 72), (12, 2, 300, 128, 96), (4, 1, 1, 80, 48), (6, 2, 3, 256, 33),
-                                             (4, 2, 700, 200, 136), (2, 1, 1000, 72, 264)])
+                                             (4, 2, 700, 200, 136), (2, 1, 1000, 72, 264), (8, 2, 8, 1024, 520), (3, 2, 40, 2056, 48),
+                                             (2, 2, 64, 320, 24)])
 def test_experts_products_over_runs_of_pairs(E, top, T, d, F, dtype, mfma):
     """Runs of unequal lengths, experts that nobody chose, more pairs than a tile holds, one token; each pair's hidden
     row and output against the plain expert of its choice."""
