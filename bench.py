@@ -366,8 +366,8 @@ def nolatar_config(shape, layers, chunk=1024):
            "mixer": {"heads": d // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
     left = {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5, "rot": rot, "mask": {"size": chunk}}
     right = {"heads": H // 2, "dim": hs, "vdim": 2 * hs, "rot": rot, "decay": [1.0 - 2.0 ** (-5 - (i % 8)) for i in range(H // 2)]}
-    side = {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": right, "left_scale": 0.6, "right_scale": 1.1}}
-    diff = {"heads": H // 2, "kv_heads": max(1, G // 2), "dim": hs, "vdim": hs, "scale": hs ** -0.5, "diff": 0.6, "rot": rot}
+    side = {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": right, "left_scale": 0.75, "right_scale": 1.25}}
+    diff = {"heads": H // 2, "kv_heads": max(1, G // 2), "dim": hs, "vdim": hs, "scale": hs ** -0.5, "diff": 0.5, "rot": rot}
     out = []
     for i in range(layers):
         kind = i % 4

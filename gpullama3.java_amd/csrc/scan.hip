@@ -8,7 +8,8 @@
 // inputs of every sequence kept in its slot; the decays and step sizes; and the read-outs' gate and unit norm.
 // Everything here is 32-bit arithmetic with accurate exp; only the last kernel's output takes the activations' type.
 // Every kernel walks a step's tokens in order from what the slot holds, and no sum depends on what else is in the
-// batch, so any cut of a sequence into steps gives the same numbers.
+// batch, so any cut of a sequence into steps gives the same numbers (a long step's recurrence runs in pieces joined
+// through their start states: the same numbers up to 32-bit rounding).
 #include "common.h"
 
 // ----------------------------------------------------------------- convolution, decays and step sizes

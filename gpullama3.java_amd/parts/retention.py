@@ -10,8 +10,9 @@ are multiplied by silu of a gate projection, and the output projection follows.
 
 One product makes q, k, v and the gate (rows stacked, padded with zero rows to a multiple of 16); its sums stay in
 32-bit, and so does everything up to the output projection's input. The recurrence is ``lib.decay_scan``
-(``csrc/scan.hip``), which the state space shares: it walks a step's tokens in order from the slot's state, so every
-cut of a sequence into steps gives the same result.
+(``csrc/scan.hip``), which the state space shares: it walks a step's tokens in order from the slot's state (a long
+step as pieces side by side, joined through their start states), so every cut of a sequence into steps gives the same
+result up to 32-bit rounding.
 """
 from __future__ import annotations
 

@@ -73,10 +73,10 @@ REORDERED = {
 # fast paths (experts' products on the matrix cores, heads of 64 and 128 with values of the keys' size)
 TILED = {
     "architecture": "Nolatar", "vocab": 640, "width": 128, "norm": {"eps": 1e-5},
-    "layers": [_parallel(_left(4, 2, 64, 64, 0.125, 10000.0, 64, 100), _right(2, 64, 64, [0.97, 0.99], 10000.0, 64), 0.6, 1.1, _moe(4, 2, 64, 128)),
+    "layers": [_parallel(_left(4, 2, 64, 64, 0.125, 10000.0, 64, 100), _right(2, 64, 64, [0.97, 0.99], 10000.0, 64), 0.75, 1.2, _moe(4, 2, 64, 128)),
                _mamba(4, 32, 64, 2, 4, 2, _moe(8, 2, 32, 32)),
-               _diff(2, 1, 64, 64, 0.125, 0.6, 250000.0, 64, _moe(4, 2, 64, 64)),
-               _diff(2, 1, 64, 64, 0.125, 0.6, 250000.0, 64, None, kv_from=2),
+               _diff(2, 1, 64, 64, 0.125, 0.45, 40000.0, 64, _moe(4, 2, 64, 64)),
+               _diff(2, 1, 64, 64, 0.125, 0.45, 40000.0, 64, None, kv_from=2),
                _parallel(_left(2, 1, 128, 128, 0.09, 50000.0, 64, 130), _right(1, 128, 128, [0.98], 50000.0, 32), 1.0, 1.0, None)],
 }
 CONFIGS = {"mixed": MIXED, "reordered": REORDERED, "tiled": TILED}
