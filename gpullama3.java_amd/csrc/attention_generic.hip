@@ -25,11 +25,11 @@
 
 #define ATT_MAX_HS 256
 
-template <typename T>
+template <typename T, typename TO>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-    int table_stride, T* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
+    int table_stride, TO* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
     int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink, int keep_first,
     int chunk, int n_v) {
   __shared__ float qs[ATT_MAX_HS];
@@ -88,11 +88,11 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     m = m_new;
   }
   }
-  T* op = out + (long)t * out_stride + (long)h * v_head_dim;
+  TO* op = out + (long)t * out_stride + (long)h * v_head_dim;
 #pragma unroll
   for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
     const int i = lane + 64 * r;
-    if (i < v_head_dim) op[i] = from_f32<T>(acc[r] / l);
+    if (i < v_head_dim) op[i] = from_f32<TO>(acc[r] / l);
   }
 }
 
@@ -101,7 +101,7 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
                                      int table_stride, void* out, long out_stride, int n_tokens, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int v_head_dim,
                                      const float* slopes, int has_sink, float sink, int keep_first, int chunk, int n_v,
-                                     hipStream_t stream) {
+                                     int out_dtype, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
               "gl3_attention_generic: null argument");
@@ -121,17 +121,17 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
               "gl3_attention_generic: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16", page_size,
               head_dim);
   dim3 grid(n_tokens, n_heads), block(64);
-  if (dtype == GL3_F32)
-    attention_generic_kernel<float><<<grid, block, 0, stream>>>(
-        (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, positions, seq_of_token, block_table,
-        table_stride, (float*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink,
-        sink, keep_first, chunk, n_v);
-  else if (dtype == GL3_BF16)
-    attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,
-        block_table, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale,
-        slopes, has_sink, sink, keep_first, chunk, n_v);
-  else GL3_REQUIRE(false, "gl3_attention_generic: unknown dtype %d", dtype);
+#define ATT_GENERIC(T, TO)                                                                                             \
+  attention_generic_kernel<T, TO><<<grid, block, 0, stream>>>(                                                         \
+      (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, positions, seq_of_token, block_table, table_stride, \
+      (TO*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink, sink,     \
+      keep_first, chunk, n_v)
+  // (the output in 32-bit beside 16-bit operands: for a caller that goes on in 32-bit with the heads' outputs)
+  if (dtype == GL3_F32 && out_dtype == GL3_F32) ATT_GENERIC(float, float);
+  else if (dtype == GL3_BF16 && out_dtype == GL3_BF16) ATT_GENERIC(bf16_t, bf16_t);
+  else if (dtype == GL3_BF16 && out_dtype == GL3_F32) ATT_GENERIC(bf16_t, float);
+  else GL3_REQUIRE(false, "gl3_attention_generic: dtypes %d -> %d are not built", dtype, out_dtype);
+#undef ATT_GENERIC
   GL3_LAUNCH_CHECK();
   return 0;
 }

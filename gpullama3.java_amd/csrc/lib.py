@@ -57,11 +57,11 @@ def _declare(lib):
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, F, F, P, P],
-        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, I, P],
         "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
         "gl3_concat_rows": [P, P, P, I, I, I, P],
         "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P, P, F, P],
-        "gl3_diff_combine": [P, L, P, L, I, I, I, I, I, F, F, F, P],
+        "gl3_diff_combine": [P, I, L, P, L, I, I, I, I, I, F, F, F, P],
         "gl3_layernorm": [P, P, P, P, P, I, I, I, F, P],
         "gl3_layernorm_add": [P, P, P, P, I, I, F, P, I, P],
         "gl3_cast_rows": [P, P, I, L, P],
@@ -413,8 +413,8 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
     _dev(block_table, "block_table", torch.int32)
     T = q.shape[0]
-    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim or out.dtype != q.dtype:
-        raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim or out.dtype not in (q.dtype, torch.float32):
+        raise KernelError(f"attention: q {tuple(q.shape)} {q.dtype} for {n_heads} heads of {head_dim}, out {out.dtype}")
     vd = head_dim if v_head_dim is None else int(v_head_dim)
     if out.shape != (T, n_heads * vd) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
@@ -432,7 +432,7 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
         int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0),
-        int(keep_first or 0) if window else 0, int(chunk or 0), n_v, _stream()),
+        int(keep_first or 0) if window else 0, int(chunk or 0), n_v, _code(out, "out"), _stream()),
         "attention_generic")
 
 
@@ -556,12 +556,15 @@ def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, g
 
 def diff_combine(att, out, H, D, dim, lam, eps, mult):
     """``att`` [T, 2 H D]: head by head the output under the first score map and under the second; ``out`` [T, H D] =
-    (a1 - lam * a2) / rms over the head's first ``dim`` elements (what lies behind them holds zeros) * mult."""
-    _dev(att, "att", contiguous=False); _dev(out, "out", att.dtype, contiguous=False)
+    (a1 - lam * a2) / rms over the head's first ``dim`` elements (what lies behind them holds zeros) * mult. ``att`` has
+    ``out``'s type or is float32."""
+    _dev(att, "att", contiguous=False); _dev(out, "out", contiguous=False)
+    if att.dtype not in (out.dtype, torch.float32):
+        raise KernelError(f"diff_combine: {att.dtype} -> {out.dtype}")
     T = att.shape[0]
     if att.dim() != 2 or att.stride(1) != 1 or att.shape[1] < 2 * H * D or out.shape != (T, H * D) or out.stride(1) != 1:
         raise KernelError(f"diff_combine: {tuple(att.shape)} -> {tuple(out.shape)} for {H} heads of {D}")
-    _check(library().gl3_diff_combine(_ptr(att), att.stride(0), _ptr(out), out.stride(0), _code(att, "att"), T, int(H), int(D),
+    _check(library().gl3_diff_combine(_ptr(att), _code(att, "att"), att.stride(0), _ptr(out), out.stride(0), _code(out, "out"), T, int(H), int(D),
                                       int(dim), float(lam), float(eps), float(mult), _stream()), "diff_combine")
 
 

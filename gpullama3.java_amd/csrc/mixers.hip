@@ -676,36 +676,39 @@ extern "C" int gl3_head_norm_gate(const float* o, const float* w, const float* g
 // ----------------------------------------------------------------- two score maps' outputs into one
 // att [T][ld_a]: head h's output under the first map at column 2 h D, under the second at (2 h + 1) D. out [T][ld_o],
 // head h at h * D: o = a1 - lambda a2, divided by its root mean square over the head's `dim` elements (eps inside
-// the root; elements behind them are padding and hold zeros), times `mult`. One wave a (token, head).
-template <typename T>
-__global__ __launch_bounds__(64) void diff_combine_kernel(const T* __restrict__ att, long ld_a, T* __restrict__ out, long ld_o,
+// the root; elements behind them are padding and hold zeros), times `mult`. One wave a (token, head). The maps'
+// outputs may come in 32-bit where the result takes the activations' type.
+template <typename TI, typename T>
+__global__ __launch_bounds__(64) void diff_combine_kernel(const TI* __restrict__ att, long ld_a, T* __restrict__ out, long ld_o,
                                                            int H, int D, int dim, float lambda, float eps, float mult) {
   const long t = blockIdx.x;
   const int h = blockIdx.y;
-  const T* a1 = att + t * ld_a + (long)2 * h * D;
-  const T* a2 = a1 + D;
+  const TI* a1 = att + t * ld_a + (long)2 * h * D;
+  const TI* a2 = a1 + D;
   float ss = 0.f;
   for (int i = threadIdx.x; i < dim; i += 64) {
-    const float o = to_f32<T>(a1[i]) - lambda * to_f32<T>(a2[i]);
+    const float o = to_f32<TI>(a1[i]) - lambda * to_f32<TI>(a2[i]);
     ss += o * o;
   }
   const float f = mult / sqrtf(wave_sum(ss) / (float)dim + eps);
   T* op = out + t * ld_o + (long)h * D;
-  for (int i = threadIdx.x; i < D; i += 64) op[i] = from_f32<T>((to_f32<T>(a1[i]) - lambda * to_f32<T>(a2[i])) * f);
+  for (int i = threadIdx.x; i < D; i += 64) op[i] = from_f32<T>((to_f32<TI>(a1[i]) - lambda * to_f32<TI>(a2[i])) * f);
 }
 
-extern "C" int gl3_diff_combine(const void* att, long ld_a, void* out, long ld_o, int dtype, int n_tokens, int H, int D, int dim,
-                                float lambda, float eps, float mult, hipStream_t stream) {
+extern "C" int gl3_diff_combine(const void* att, int in_dtype, long ld_a, void* out, long ld_o, int dtype, int n_tokens, int H,
+                                int D, int dim, float lambda, float eps, float mult, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(att && out && n_tokens > 0 && H > 0 && H <= 65535 && D > 0 && dim > 0 && dim <= D && ld_a >= 2L * H * D &&
                   ld_o >= (long)H * D,
               "gl3_diff_combine: %d heads of %d (%d used) in rows of %ld and %ld", H, D, dim, ld_a, ld_o);
   const dim3 grid(n_tokens, H), block(64);
-  if (dtype == GL3_F32)
-    diff_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)att, ld_a, (float*)out, ld_o, H, D, dim, lambda, eps, mult);
-  else if (dtype == GL3_BF16)
-    diff_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)att, ld_a, (bf16_t*)out, ld_o, H, D, dim, lambda, eps, mult);
-  else GL3_REQUIRE(false, "gl3_diff_combine: unknown dtype %d", dtype);
+  if (in_dtype == GL3_F32 && dtype == GL3_F32)
+    diff_combine_kernel<float, float><<<grid, block, 0, stream>>>((const float*)att, ld_a, (float*)out, ld_o, H, D, dim, lambda, eps, mult);
+  else if (in_dtype == GL3_BF16 && dtype == GL3_BF16)
+    diff_combine_kernel<bf16_t, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)att, ld_a, (bf16_t*)out, ld_o, H, D, dim, lambda, eps, mult);
+  else if (in_dtype == GL3_F32 && dtype == GL3_BF16)
+    diff_combine_kernel<float, bf16_t><<<grid, block, 0, stream>>>((const float*)att, ld_a, (bf16_t*)out, ld_o, H, D, dim, lambda, eps, mult);
+  else GL3_REQUIRE(false, "gl3_diff_combine: dtypes %d -> %d are not built", in_dtype, dtype);
   GL3_LAUNCH_CHECK();
   return 0;
 }

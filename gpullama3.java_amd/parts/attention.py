@@ -246,13 +246,16 @@ class GQAAttention:
         elif pos is not None or normed:
             K.rotate_heads(qkv, ctx.positions, [(0, Hq, hs) + qk], adjacent=bool(pos is not None and pos.adjacent),
                            norms=[(self.q_norm_w, self.hs_stored)] if normed else None, norm_eps=self.qk_norm_eps or 0.0)
-        att = ctx.buffer("attn_out", (T, Hq * vd), self.dtype)
+        att_dtype = self.dtype
+        if self.diff is not None and ops.attention_kernel(ctx, self.dtype, k_cache.shape[2], Hq, Kq, hs, self.scale, vd) == "generic":
+            att_dtype = torch.float32      # the maps' outputs stay in 32-bit up to their difference, where the kernel can write them so
+        att = ctx.buffer("attn_out", (T, Hq * vd), att_dtype)
         ops.attention(ctx, qkv, k_cache, v_cache, table, att, Hq, Kq, hs, self.window, self.scale, v_head_dim=vd,
                       slopes=self.slopes, sink=self.sink, keep_first=self.keep_first, chunk=self.chunk,
                       n_v_heads=Kh if self.maps > 1 else None)
         if self.diff is not None:
             # the two maps' outputs of every head into one: a1 - lambda a2, a unit norm per head, the factor 1 - offset
-            both, att = att, ctx.buffer("attn_maps_joined", (T, H * vd), self.dtype)
+            both, att = att, ctx.buffer("attn_maps_joined", (T, H * vd), self.dtype)      # (the activations' type again)
             K.diff_combine(both, att, H, vd, self.vd_stored, self.diff_lambda, self.diff.norm_eps, 1.0 - self.diff.offset)
         if vpos is not None or self.gated:
             # every head's output turned back by the query's position, then times the head's gate

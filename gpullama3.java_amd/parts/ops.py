@@ -466,6 +466,21 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     return qkv
 
 
+def attention_kernel(ctx, dtype, page, n_heads, n_kv, head_dim, scale, v_head_dim=None):
+    """Which kernel a step's attention runs on: "decode" or "prefill" (the matrix cores: bfloat16, values of the keys'
+    size, head sizes and pages that they are built for; their output has the activations' type) or "generic" (any
+    sizes; its output may be float32 beside bfloat16 operands)."""
+    disabled = _off(ctx)
+    if dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):
+        if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
+                and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
+            return "decode"
+        if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
+                and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
+            return "prefill"
+    return "generic"
+
+
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale, v_head_dim=None,
               slopes=None, sink=None, keep_first=0, chunk=None, n_v_heads=None):
     """``v_head_dim``: the values' size (None: the keys'); ``slopes``: float32 [H], a bias of -slopes[h] * distance
@@ -474,29 +489,26 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
     keys of its own run of n positions only; ``n_v_heads``: value heads where several score maps share them
     (``lib.attention_generic``)."""
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
-    disabled = _off(ctx)
     extras = dict(slopes=slopes, sink=sink)
     extras["keep_first"] = int(keep_first or 0) if window else 0
     extras.update(chunk=int(chunk or 0), n_v_heads=n_v_heads)
-    if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
-        if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
-                and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
-            T = q.shape[0]
-            splits = K.decode_splits(T, n_heads, n_kv, min(ctx.kv_len_hint, chunk) if chunk else ctx.kv_len_hint, head_dim)
-            part_o = part_ml = None
-            if splits > 1:
-                part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
-                part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
-            own = getattr(ctx, "token_tables", {}).get(block_table.data_ptr())    # (made with the step's token facts)
-            if own is not None:
-                return K.attention_decode(q, k_cache, v_cache, ctx.positions, None, own, out, n_heads, n_kv, head_dim, page,
-                                          window, scale, splits, part_o, part_ml, **extras)
-            return K.attention_decode(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads,
-                                      n_kv, head_dim, page, window, scale, splits, part_o, part_ml, **extras)
-        if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
-                and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
-            return K.attention_prefill(q, k_cache, v_cache, ctx.cu_seqlens, ctx.kv_before, block_table, out,
-                                       ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
-                                       seq_rows=getattr(ctx, "seq_rows", None), **extras)
+    kernel = attention_kernel(ctx, q.dtype, page, n_heads, n_kv, head_dim, scale, v_head_dim)
+    if kernel == "decode":
+        T = q.shape[0]
+        splits = K.decode_splits(T, n_heads, n_kv, min(ctx.kv_len_hint, chunk) if chunk else ctx.kv_len_hint, head_dim)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
+            part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
+        own = getattr(ctx, "token_tables", {}).get(block_table.data_ptr())    # (made with the step's token facts)
+        if own is not None:
+            return K.attention_decode(q, k_cache, v_cache, ctx.positions, None, own, out, n_heads, n_kv, head_dim, page,
+                                      window, scale, splits, part_o, part_ml, **extras)
+        return K.attention_decode(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads,
+                                  n_kv, head_dim, page, window, scale, splits, part_o, part_ml, **extras)
+    if kernel == "prefill":
+        return K.attention_prefill(q, k_cache, v_cache, ctx.cu_seqlens, ctx.kv_before, block_table, out,
+                                   ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
+                                   seq_rows=getattr(ctx, "seq_rows", None), **extras)
     return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
                                head_dim, page, window, scale, v_head_dim=v_head_dim, **extras)

@@ -70,13 +70,15 @@ REORDERED = {
                _mamba(2, 40, 33, 2, 5, 2, _moe(2, 2, 20, 20))],
 }
 # head sizes that the matrix cores' kernels are built for, widths in whole tiles: what a bfloat16 engine runs on its
-# fast paths (experts' products on the matrix cores, heads of 64 and 128 with values of the keys' size)
+# fast paths (experts' products on the matrix cores, heads of 64 and 128 with values of the keys' size). The offset of
+# the differential layers keeps their lambda (0.39 and 1.28 with these weights) away from 1, where the two maps cancel
+# and a bfloat16 engine's rounding of the maps' outputs is all that is left of a head
 TILED = {
     "architecture": "Nolatar", "vocab": 640, "width": 128, "norm": {"eps": 1e-5},
     "layers": [_parallel(_left(4, 2, 64, 64, 0.125, 10000.0, 64, 100), _right(2, 64, 64, [0.97, 0.99], 10000.0, 64), 0.75, 1.2, _moe(4, 2, 64, 128)),
                _mamba(4, 32, 64, 2, 4, 2, _moe(8, 2, 32, 32)),
-               _diff(2, 1, 64, 64, 0.125, 0.45, 40000.0, 64, _moe(4, 2, 64, 64)),
-               _diff(2, 1, 64, 64, 0.125, 0.45, 40000.0, 64, None, kv_from=2),
+               _diff(2, 1, 64, 64, 0.125, 0.7, 40000.0, 64, _moe(4, 2, 64, 64)),
+               _diff(2, 1, 64, 64, 0.125, 0.7, 40000.0, 64, None, kv_from=2),
                _parallel(_left(2, 1, 128, 128, 0.09, 50000.0, 64, 130), _right(1, 128, 128, [0.98], 50000.0, 32), 1.0, 1.0, None)],
 }
 CONFIGS = {"mixed": MIXED, "reordered": REORDERED, "tiled": TILED}

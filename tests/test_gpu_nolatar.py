@@ -107,12 +107,12 @@ def paged(k, v, page, dtype):
     return (dev(tile_keys(kc), TD[dtype]), dev(tile_values(vc), TD[dtype]), i32(np.arange(1, n + 1)[None]))
 
 
-def attention_on_gpu(q, k, v, positions, dtype, chunk, scale, maps=1, page=64):
+def attention_on_gpu(q, k, v, positions, dtype, chunk, scale, maps=1, page=64, out_dtype=None):
     """q [T, H * maps, D], k [S, G * maps, D], v [S, G, Dv] -> [T, H * maps, Dv] from the kernel for any sizes."""
     from gpullama3_java_amd.csrc import lib as K
     T, Hq, D = q.shape
     kc, vc, table = paged(k, v, page, dtype)
-    out = torch.zeros(T, Hq * v.shape[2], dtype=TD[dtype], device=DEV)
+    out = torch.zeros(T, Hq * v.shape[2], dtype=TD[out_dtype or dtype], device=DEV)
     K.attention_generic(dev(q.reshape(T, Hq * D), TD[dtype]), kc, vc, i32(positions), i32([0] * T), table, out, Hq, k.shape[1],
                         D, page, None, scale, v_head_dim=v.shape[2], chunk=chunk or 0, n_v_heads=v.shape[1] if maps > 1 else None)
     return host(out).reshape(T, Hq, v.shape[2])
@@ -233,6 +233,14 @@ def test_two_score_maps_over_the_same_values(H, G, D, Dv, dtype):
     for m in range(2):
         ref = plain_attention_at(q[positions][:, :, m], k[:, :, m], v, positions, None, 0.2)
         np.testing.assert_allclose(got[:, :, m], ref, atol=2e-4 if dtype == "float32" else 0.05, err_msg=f"map {m}")
+    if dtype == "bfloat16":
+        # the same kernel writes its output in 32-bit beside 16-bit operands: what it rounded before is what differs
+        wide = attention_on_gpu(q[positions].reshape(-1, H * 2, D), k.reshape(S, G * 2, D), v, positions, dtype, None, 0.2, maps=2,
+                                out_dtype="float32").reshape(got.shape)
+        np.testing.assert_array_equal(torch.tensor(wide).to(torch.bfloat16).float().numpy(), got)
+        for m in range(2):
+            ref = plain_attention_at(q[positions][:, :, m], k[:, :, m], v, positions, None, 0.2)
+            np.testing.assert_allclose(wide[:, :, m], ref, atol=2e-4, err_msg=f"map {m} in 32-bit")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -248,6 +256,14 @@ def test_the_maps_outputs_joined(dtype):
     got = host(out).reshape(T, H, Dpad)
     np.testing.assert_allclose(got[..., :D], ref, atol=1e-5 if dtype == "float32" else 0.02)
     assert not got[..., D:].any()
+    if dtype == "bfloat16":
+        # the maps' outputs in 32-bit, the result in bfloat16; two maps that nearly cancel (lambda close to 1 over
+        # nearly equal outputs) keep what 16-bit inputs would lose
+        b = a.copy()
+        b[:, :, 1, :D] = b[:, :, 0, :D] * (1 + 1e-3 * rng.standard_normal((T, H, D)))
+        K.diff_combine(dev(b.reshape(T, -1)), out, H, Dpad, D, 0.999, 1e-5, 0.45)
+        ref = P.rms_unit(b[:, :, 0, :D] - 0.999 * b[:, :, 1, :D], 1e-5) * 0.45
+        np.testing.assert_allclose(host(out).reshape(T, H, Dpad)[..., :D], ref, atol=0.02)
 
 
 # ----------------------------------------------------------------- the state space's and the retention's kernels
@@ -751,7 +767,7 @@ def random_config(seed):
     n_layers = int(rng.integers(2, 7))
 
     def rot(dim):
-        return {"base": pick([100.0, 10000.0, 300000.0, 1e6]), "dims": pick([d for d in (2, 4, 8, 16, 24, 32, 48, 64, 96, 128) if d <= dim])}
+        return {"base": pick([100.0, 10000.0, 250000.0, 1e6]), "dims": pick([d for d in (2, 4, 8, 16, 24, 32, 48, 64, 96, 128) if d <= dim])}
 
     layers, owners = [], []
     for i in range(n_layers):
@@ -776,19 +792,19 @@ def random_config(seed):
             rh = pick([1, 2, 3, 4])
             right = {"heads": rh, "dim": rdim, "vdim": pick([8, 16, 24, 40, 64]), "rot": rot(rdim),
                      "decay": [float(1 - 2.0 ** -rng.integers(2, 11)) for _ in range(rh)]}
-            m = {"left": left, "right": right, "left_scale": float(pick([0.5, 0.65, 1.0, 1.5])), "right_scale": float(pick([0.4, 1.0, 1.15]))}
+            m = {"left": left, "right": right, "left_scale": float(pick([0.5, 0.6, 1.0, 1.5])), "right_scale": float(pick([0.4, 1.0, 1.1]))}
         else:
             if owners and rng.random() < 0.45:
                 j = pick(owners)
                 o = layers[j]["mixer"]
                 m = {"heads": o["kv_heads"] * pick([1, 2, 3]), "kv_heads": o["kv_heads"], "dim": o["dim"], "vdim": o["vdim"],
-                     "scale": float(pick([0.1, 0.15, 0.3])), "diff": float(pick([0.2, 0.65, 0.8])), "rot": dict(o["rot"]), "kv_from": j}
+                     "scale": float(pick([0.1, 0.15, 0.3])), "diff": float(pick([0.2, 0.6, 0.8])), "rot": dict(o["rot"]), "kv_from": j}
             else:
                 heads = pick([1, 2, 3, 4, 6])
                 dim = pick([8, 16, 24, 32, 48, 64])
                 m = {"heads": heads, "kv_heads": pick([k for k in (1, 2, 3, 6) if heads % k == 0]), "dim": dim,
                      "vdim": pick([8, 16, 24, 32, 48, 96]), "scale": float(pick([0.1, 0.15, dim ** -0.5])),
-                     "diff": float(pick([0.2, 0.5, 0.65, 0.8])), "rot": rot(dim)}
+                     "diff": float(pick([0.2, 0.5, 0.6, 0.8])), "rot": rot(dim)}
                 owners.append(i)
         layers.append({"type": kind, "mixer": m, "mlp": mlp})
     return {"architecture": "Nolatar", "vocab": int(rng.integers(50, 700)), "width": width, "norm": {"eps": pick([1e-5, 1e-6])},
