@@ -250,64 +250,84 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __r
 }
 
 // For few rows (decode steps: an expert's run is a handful of pairs, and the time goes into reading its weights
-// once): a block of 8 waves works a tile of 16 rows of one run x 16 columns, wave w a slice of K (the slices follow
-// from K alone), 32 k a step with v_mfma_f32_16x16x32_bf16: a lane holds 8 consecutive k of a row of A and of a row
-// of W, read 16 bytes at a time, four steps in flight. The slices' sums are added in their order through shared memory.
+// once): a block of 8 waves works a tile of 16 G rows of one run x 16 columns (G = 1, 2 or 4 by the runs' mean length,
+// so that a run is mostly one tile and its weights are read once), wave w a slice of K (the slices follow from K
+// alone), 32 k a step with v_mfma_f32_16x16x32_bf16: a lane holds 8 consecutive k of a row of A and of a row of W,
+// read 16 bytes at a time, four steps in flight. The slices' sums are added in their order through shared memory.
 typedef __bf16 bf16x8_few_t __attribute__((ext_vector_type(8)));
 #define EF_WAVES 8
-#define EF_TM 16
 #define EF_TN 16
-template <typename TO>
+template <typename TO, int G>
 __global__ __launch_bounds__(EF_WAVES * 64) void expert_gemm_few_kernel(const bf16_t* __restrict__ A, long lda, int a_div,
                                                                         const bf16_t* __restrict__ W, int N, int K,
                                                                         const int* __restrict__ offsets,
                                                                         const int* __restrict__ sorted, int E, int n_rows,
                                                                         TO* __restrict__ out, long ldo, int act) {
-  __shared__ int rows[EF_TM];
-  __shared__ float part[EF_WAVES][EF_TM][EF_TN + 1];
+  constexpr int TM = 16 * G;
+  __shared__ int rows[TM];
+  __shared__ float part[EF_WAVES][TM][EF_TN + 1];
   int e, lo, hi;
-  if (!expert_tile(offsets, E, n_rows, EF_TM, blockIdx.x, &e, &lo, &hi)) return;
-  const int m = hi - lo < EF_TM ? hi - lo : EF_TM;
-  if (threadIdx.x < EF_TM) rows[threadIdx.x] = threadIdx.x < m ? (sorted ? sorted[lo + threadIdx.x] : lo + threadIdx.x) : -1;
+  if (!expert_tile(offsets, E, n_rows, TM, blockIdx.x, &e, &lo, &hi)) return;
+  const int m = hi - lo < TM ? hi - lo : TM;
+  if (threadIdx.x < TM) rows[threadIdx.x] = (int)threadIdx.x < m ? (sorted ? sorted[lo + threadIdx.x] : lo + threadIdx.x) : -1;
   __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int li = lane & 15, kg = (lane >> 4) * 8;
   const int n = blockIdx.y * EF_TN + li;
   const int per = ((K + 31) / 32 + EF_WAVES - 1) / EF_WAVES * 32;       // this wave's slice of K
   const int k_lo = wave * per, k_hi = k_lo + per < K ? k_lo + per : K;
-  const int row = rows[li];
+  const int groups = (m + 15) / 16;
   const bf16_t* wp = W + ((long)e * N + (n < N ? n : N - 1)) * K + kg;
-  const bf16_t* ap = A + (long)(row >= 0 ? row / a_div : rows[0] / a_div) * lda + kg;
+  const bf16_t* ap[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int row = rows[g * 16 + li];                  // (rows beyond the run read the run's first row; their results are dropped)
+    ap[g] = A + (long)((row >= 0 ? row : rows[0]) / a_div) * lda + kg;
+  }
   const bf16x8_few_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) acc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
   int k0 = k_lo;
   for (; k0 + 128 <= k_hi; k0 += 128) {
-    bf16x8_few_t a[4], b[4];
+    bf16x8_few_t a[4][G], b[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       b[u] = *reinterpret_cast<const bf16x8_few_t*>(wp + k0 + 32 * u);
-      a[u] = *reinterpret_cast<const bf16x8_few_t*>(ap + k0 + 32 * u);
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        if (g < groups) a[u][g] = *reinterpret_cast<const bf16x8_few_t*>(ap[g] + k0 + 32 * u);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], acc, 0, 0, 0);
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        if (g < groups) acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][g], b[u], acc[g], 0, 0, 0);
   }
   for (; k0 < k_hi; k0 += 32) {
     const bool in = k0 + kg < k_hi;                     // (K is a multiple of 8: a lane's 8 k lie inside or outside)
     const bf16x8_few_t b = in ? *reinterpret_cast<const bf16x8_few_t*>(wp + k0) : zero;
-    const bf16x8_few_t a = in ? *reinterpret_cast<const bf16x8_few_t*>(ap + k0) : zero;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-  }
-  // a lane holds column li of rows 4 (lane / 16) .. + 3
 #pragma unroll
-  for (int i = 0; i < 4; ++i) part[wave][(lane >> 4) * 4 + i][li] = acc[i];
+    for (int g = 0; g < G; ++g) {
+      if (g < groups) {
+        const bf16x8_few_t a = in ? *reinterpret_cast<const bf16x8_few_t*>(ap[g] + k0) : zero;
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[g], 0, 0, 0);
+      }
+    }
+  }
+  // a lane holds column li of rows 4 (lane / 16) .. + 3 of every group
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][g * 16 + (lane >> 4) * 4 + i][li] = acc[g][i];
   __syncthreads();
-  if (threadIdx.x < EF_TM * EF_TN) {
-    const int r = threadIdx.x / EF_TN, c = threadIdx.x % EF_TN;
+  for (int idx = threadIdx.x; idx < m * EF_TN; idx += EF_WAVES * 64) {
+    const int r = idx / EF_TN, c = idx % EF_TN;
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < EF_WAVES; ++w) sum += part[w][r][c];
     const int nc = blockIdx.y * EF_TN + c;
-    if (rows[r] >= 0 && nc < N) out[(long)rows[r] * ldo + nc] = from_f32<TO>(gl3_expert_act(sum, act));
+    if (nc < N) out[(long)rows[r] * ldo + nc] = from_f32<TO>(gl3_expert_act(sum, act));
   }
 }
 
@@ -428,10 +448,11 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
               "gl3_expert_gemm: runs and their pairs come together; without them one expert takes every row");
   GL3_REQUIRE(act >= 0 && act <= 3, "gl3_expert_gemm: unknown activation %d", act);
   GL3_REQUIRE((N + 63) / 64 <= 65535, "gl3_expert_gemm: %d columns exceed the grid", N);
+  const int e_eff = offsets ? E : 1;
   // many rows (an expert's run fills tiles of 128): the tiled kernel
   if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 8 == 0 && K >= 8 && lda % 8 == 0 &&
       (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0) &&
-      n_rows >= 64 * (offsets ? E : 1) && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
+      n_rows > 64 * e_eff && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
     const dim3 grid((n_rows + ET_BM - 1) / ET_BM + (offsets ? E : 0), (N + ET_BN - 1) / ET_BN), block(512);
     if (out_dtype == GL3_BF16)
       expert_gemm_tiled_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
@@ -442,17 +463,21 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
     GL3_LAUNCH_CHECK();
     return 0;
   }
-  // few rows (an expert's run is a tile of 16 or two): the kernel that reads each weight row in long pieces, K in slices
+  // few rows (an expert's run is a tile or two): the kernel that reads each weight row in long pieces, K in slices
   if (use_mfma && a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && K % 8 == 0 && lda % 8 == 0 &&
       (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0) &&
-      n_rows <= 32 * (offsets ? E : 1) && (N + EF_TN - 1) / EF_TN <= 65535 && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
-    const dim3 grid((n_rows + EF_TM - 1) / EF_TM + (offsets ? E : 0), (N + EF_TN - 1) / EF_TN), block(EF_WAVES * 64);
-    if (out_dtype == GL3_BF16)
-      expert_gemm_few_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                 sorted, E, n_rows, (bf16_t*)out, ldo, act);
-    else
-      expert_gemm_few_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                sorted, E, n_rows, (float*)out, ldo, act);
+      n_rows <= 64 * e_eff && (N + EF_TN - 1) / EF_TN <= 65535 && (out_dtype == GL3_BF16 || out_dtype == GL3_F32)) {
+    const int G = n_rows <= 16 * e_eff ? 1 : n_rows <= 32 * e_eff ? 2 : 4;      // by the runs' mean length
+    const dim3 grid((n_rows + 16 * G - 1) / (16 * G) + (offsets ? E : 0), (N + EF_TN - 1) / EF_TN), block(EF_WAVES * 64);
+#define EF_LAUNCH(TO, G)                                                                                                \
+  expert_gemm_few_kernel<TO, G><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets, \
+                                                            sorted, E, n_rows, (TO*)out, ldo, act)
+    if (out_dtype == GL3_BF16) {
+      if (G == 1) EF_LAUNCH(bf16_t, 1); else if (G == 2) EF_LAUNCH(bf16_t, 2); else EF_LAUNCH(bf16_t, 4);
+    } else {
+      if (G == 1) EF_LAUNCH(float, 1); else if (G == 2) EF_LAUNCH(float, 2); else EF_LAUNCH(float, 4);
+    }
+#undef EF_LAUNCH
     GL3_LAUNCH_CHECK();
     return 0;
   }

@@ -494,7 +494,7 @@ def test_router_choice_ties_weights_and_runs():
 @pytest.mark.parametrize("dtype, mfma", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
 @pytest.mark.parametrize("E, top, T, d, F", [(5, 2, 90, 96, 40), (3, 3, 7, 64, 72), (11, 2, 300, 128, 88), (4, 1, 1, 80, 48), (6, 2, 3, 256, 33),
                                              (4, 2, 700, 200, 136), (2, 1, 1000, 72, 264), (8, 2, 8, 1024, 520), (3, 2, 40, 2056, 48),
-                                             (2, 2, 64, 320, 24)])
+                                             (2, 2, 64, 320, 24), (4, 2, 50, 256, 136), (4, 2, 100, 192, 64), (2, 1, 24, 136, 72)])
 def test_experts_products_over_runs_of_pairs(E, top, T, d, F, dtype, mfma):
     """Runs of unequal lengths, experts that nobody chose, more pairs than a tile holds, one token; each pair's hidden
     row and output against the plain expert of its choice."""
