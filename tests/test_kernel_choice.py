@@ -135,3 +135,21 @@ def test_strips_slices_and_pieces_of_the_products_of_few_rows():
     assert ops.gated_on_whole_lines(torch.empty(2 * 8192, 8, dtype=torch.bfloat16))
     assert not ops.gated_on_whole_lines(torch.empty(2 * 320, 8, dtype=torch.bfloat16))
     assert not ops.gated_on_whole_lines(torch.empty(2 * 8192, 8, dtype=torch.bfloat16), frozenset({"widefold"}))
+
+
+def test_a_long_step_s_recurrence_is_cut_by_its_shape():
+    # a prompt of 2,048 tokens: about a thousand (sequence, piece, head) blocks, pieces of whole rounds of 16 tokens
+    assert lib.scan_piece_len(2048, 1, 32) == 64 and lib.scan_piece_len(2048, 1, 16) == 32
+    assert lib.scan_piece_len(4096, 8, 32) == 1024 and lib.scan_piece_len(512, 8, 32) == 128
+    # decode steps and short prompts run in one piece, and need no scratch
+    for n in (1, 2, 16, 32):
+        assert lib.scan_piece_len(n, 1, 4) == 0 and lib.scan_pieces_floats(n, 64, 4, 128, 64) == 0
+    assert lib.scan_piece_len(33, 1, 4) == 32
+    for max_len in (33, 100, 777, 5000, 100000):
+        for B, H in ((1, 1), (1, 24), (3, 6), (16, 32), (200, 8)):
+            piece = lib.scan_piece_len(max_len, B, H)
+            assert piece == 0 or (piece % 16 == 0 and 32 <= piece < max_len)
+            if piece:
+                pieces = -(-max_len // piece)
+                assert pieces >= 2 and lib.scan_pieces_floats(max_len, B, H, 48, 32) == B * pieces * H * (48 * 32 + 1)
+                assert B * pieces * H <= 2 * max(lib.SCAN_PIECE_BLOCKS, B * H * 2)        # (the scratch stays bounded)
