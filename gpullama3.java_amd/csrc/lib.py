@@ -68,7 +68,7 @@ def _declare(lib):
         "gl3_ssm_prep": [P, L, I, I, I, I, I, I, P, P, I, P, P, P, L, L, P, P, P, P, P, P],
         "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P, L, I, I, P],
         "gl3_group_norm_gate": [P, P, L, I, P, I, P, L, I, P, F, I, I, I, I, P, I, P],
-        "gl3_route": [P, I, I, I, P, P, P, P, P],
+        "gl3_route": [P, I, I, I, P, P, P, P, I, P],
         "gl3_expert_gemm": [P, I, L, I, P, I, I, I, I, P, P, I, P, I, L, I, I, P],
         "gl3_route_combine": [P, P, I, I, I, P, I, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
@@ -735,20 +735,26 @@ def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=Fal
 
 
 EXPERT_ACTIVATIONS = {None: 0, "gelu": 1, "gelu_tanh": 2, "silu": 3}
+ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS = 16, 1024      # as csrc/routed.hip has them
 
 
-def route(logits, top, idx, wts, offsets, pairs):
+def route(logits, top, idx, wts, offsets, pairs, always=False):
     """Router logits [T, E] float32 -> the ``top`` largest per token (``idx`` [T, top] int32, the lower number wins a
     tie) with the softmax over them alone (``wts`` [T, top]); and the (token, choice) pairs ordered by expert:
-    ``offsets`` [E + 1] int32, ``pairs`` [T top] int32 (pair t * top + j)."""
+    ``offsets`` [E + 1] int32, ``pairs`` [T top] int32 (pair t * top + j). ``always``: every token has one more pair
+    behind its choices, with expert number E and weight 1 (``idx`` and ``wts`` [T, top + 1], ``offsets`` [E + 2],
+    ``pairs`` [T (top + 1)])."""
     _dev(logits, "logits", torch.float32)
     T, E = logits.shape
-    for t, name, shape, dt in ((idx, "idx", (T, top), torch.int32), (wts, "wts", (T, top), torch.float32),
-                               (offsets, "offsets", (E + 1,), torch.int32), (pairs, "pairs", (T * top,), torch.int32)):
+    more = 1 if always else 0
+    for t, name, shape, dt in ((idx, "idx", (T, top + more), torch.int32), (wts, "wts", (T, top + more), torch.float32),
+                               (offsets, "offsets", (E + more + 1,), torch.int32),
+                               (pairs, "pairs", (T * (top + more),), torch.int32)):
         _dev(t, name, dt)
         if tuple(t.shape) != shape:
             raise KernelError(f"route: {name} {tuple(t.shape)}, expected {shape}")
-    _check(library().gl3_route(_ptr(logits), T, E, int(top), _ptr(idx), _ptr(wts), _ptr(offsets), _ptr(pairs), _stream()), "route")
+    _check(library().gl3_route(_ptr(logits), T, E, int(top), _ptr(idx), _ptr(wts), _ptr(offsets), _ptr(pairs),
+                               E if always else -1, _stream()), "route")
 
 
 def expert_gemm(a, w, out, act=None, offsets=None, pairs=None, a_div=1, mfma=True):

@@ -13,8 +13,9 @@
 // logits [T][E] float. The `top` largest (the lower number wins a tie) -> idx [T][top]; their weights are the softmax
 // over the chosen logits alone -> wts [T][top]. One thread a token.
 __device__ __forceinline__ void route_choose(const float* __restrict__ logits, int t, int E, int top, int* idx,
-                                             float* __restrict__ wts) {
+                                             float* __restrict__ wts, int always) {
   const float* z = logits + (long)t * E;
+  const int stride = top + (always >= 0 ? 1 : 0);
   int chosen[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
   for (int j = 0; j < top; ++j) {
@@ -39,15 +40,19 @@ __device__ __forceinline__ void route_choose(const float* __restrict__ logits, i
     sum += val[j];
   }
   for (int j = 0; j < top; ++j) {
-    idx[(long)t * top + j] = chosen[j];
-    wts[(long)t * top + j] = val[j] / sum;
+    idx[(long)t * stride + j] = chosen[j];
+    wts[(long)t * stride + j] = val[j] / sum;
+  }
+  if (always >= 0) {                     // one more pair per token: the expert that every token passes, with weight 1
+    idx[(long)t * stride + top] = always;
+    wts[(long)t * stride + top] = 1.0f;
   }
 }
 
 __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ logits, int T, int E, int top,
-                                                         int* __restrict__ idx, float* __restrict__ wts) {
+                                                         int* __restrict__ idx, float* __restrict__ wts, int always) {
   const int t = blockIdx.x * 64 + threadIdx.x;
-  if (t < T) route_choose(logits, t, E, top, idx, wts);
+  if (t < T) route_choose(logits, t, E, top, idx, wts, always);
 }
 
 // ----------------------------------------------------------------- pairs ordered by expert
@@ -84,27 +89,32 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict_
 // Both in one launch for a step of at most 1024 tokens (a thread a token, then the block orders the pairs).
 __global__ __launch_bounds__(1024) void route_few_kernel(const float* __restrict__ logits, int T, int E, int top,
                                                           int* idx, float* __restrict__ wts,
-                                                          int* __restrict__ offsets, int* __restrict__ sorted) {
-  if ((int)threadIdx.x < T) route_choose(logits, threadIdx.x, E, top, idx, wts);
+                                                          int* __restrict__ offsets, int* __restrict__ sorted, int always) {
+  if ((int)threadIdx.x < T) route_choose(logits, threadIdx.x, E, top, idx, wts, always);
   __threadfence_block();
   __syncthreads();
-  route_order(idx, T * top, E, offsets, sorted);
+  const int more = always >= 0 ? 1 : 0;
+  route_order(idx, T * (top + more), E + more, offsets, sorted);
 }
 
+// `always` (-1: none): the number E of one more expert behind the router's, which every token passes with weight 1; idx
+// and wts then have top + 1 entries a token, offsets E + 2.
 extern "C" int gl3_route(const float* logits, int n_tokens, int E, int top, int* idx, float* wts, int* offsets, int* sorted,
-                         hipStream_t stream) {
+                         int always, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(logits && idx && wts && offsets && sorted, "gl3_route: null argument");
-  GL3_REQUIRE(n_tokens > 0 && E >= 1 && E <= ROUTE_MAX_EXPERTS && top >= 1 && top <= ROUTE_MAX_TOP && top <= E,
+  const int more = always >= 0 ? 1 : 0;
+  GL3_REQUIRE(n_tokens > 0 && E >= 1 && E + more <= ROUTE_MAX_EXPERTS && top >= 1 && top <= ROUTE_MAX_TOP && top <= E,
               "gl3_route: the %d largest of %d experts (at most %d of %d)", top, E, ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS);
+  GL3_REQUIRE(always < 0 || always == E, "gl3_route: the expert that every token passes is number %d, not %d", E, always);
   if (n_tokens <= 64) {
-    route_few_kernel<<<dim3(1), dim3(1024), 0, stream>>>(logits, n_tokens, E, top, idx, wts, offsets, sorted);
+    route_few_kernel<<<dim3(1), dim3(1024), 0, stream>>>(logits, n_tokens, E, top, idx, wts, offsets, sorted, always);
     GL3_LAUNCH_CHECK();
     return 0;
   }
-  route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts);
+  route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts, always);
   GL3_LAUNCH_CHECK();
-  route_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(idx, n_tokens * top, E, offsets, sorted);
+  route_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(idx, n_tokens * (top + more), E + more, offsets, sorted);
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -35,6 +35,7 @@ class RoutedFeedForward:
                 raise ValueError(f"activation {e.activation!r} is not built ({sorted(k for k in K.EXPERT_ACTIVATIONS if k)})")
         self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.w_router = self.w_up = self.w_down = self.s_up = self.s_down = None
+        self.merged = False
 
     def _expert_names(self, e):
         return self.names["expert_up"].format(e=e), self.names["expert_down"].format(e=e)
@@ -51,14 +52,24 @@ class RoutedFeedForward:
 
     def load(self, weights):
         ups, downs = zip(*[[weights[n] for n in self._expert_names(e)] for e in range(self.E)])
+        ups, downs = list(ups), list(downs)
+        # a shared expert of the experts' own form rides with them as expert number E that every token passes: its
+        # products are part of the experts' launches
+        self.merged = (self.shared is not None and self.shared.intermediate == self.F and self.shared.activation == self.act
+                       and self.top < K.ROUTE_MAX_TOP and self.E < K.ROUTE_MAX_EXPERTS)
+        if self.merged:
+            ups.append(weights[self.names["shared_up"]])
+            downs.append(weights[self.names["shared_down"]])
         # one array per kind, expert after expert; the stored names stay addressable as views
-        self.w_up = torch.stack(list(ups)).contiguous()
-        self.w_down = torch.stack(list(downs)).contiguous()
+        self.w_up = torch.stack(ups).contiguous()
+        self.w_down = torch.stack(downs).contiguous()
         for e in range(self.E):
             up, down = self._expert_names(e)
             weights[up], weights[down] = self.w_up[e], self.w_down[e]
         self.w_router = weights[self.names["router"]]
-        if self.shared is not None:
+        if self.merged:
+            weights[self.names["shared_up"]], weights[self.names["shared_down"]] = self.w_up[self.E], self.w_down[self.E]
+        elif self.shared is not None:
             self.s_up = weights[self.names["shared_up"]].contiguous().unsqueeze(0)
             self.s_down = weights[self.names["shared_down"]].contiguous().unsqueeze(0)
 
@@ -68,22 +79,24 @@ class RoutedFeedForward:
         if isinstance(h, ops.Normed):
             h = h.materialize()
         T, d, E, top, F = h.shape[0], self.d, self.E, self.top, self.F
+        more = 1 if self.merged else 0            # pairs a token beyond its choices
+        per = top + more
         mfma = "mfma" not in ops._off(ctx)
         logits = ctx.buffer("router_logits", (T, E), torch.float32)
         ops.linear(h, self.w_router, logits, ops.EPI_STORE, ctx)
-        idx = ctx.buffer("router_choice", (T, top), torch.int32)
-        wts = ctx.buffer("router_weights", (T, top), torch.float32)
-        offsets = ctx.buffer("router_runs", (E + 1,), torch.int32)
-        pairs = ctx.buffer("router_pairs", (T * top,), torch.int32)
-        K.route(logits, top, idx, wts, offsets, pairs)
-        hidden = ctx.buffer("experts_hidden", (T * top, F), self.dtype)
-        K.expert_gemm(h, self.w_up, hidden, act=self.act, offsets=offsets, pairs=pairs, a_div=top, mfma=mfma)
-        outs = ctx.buffer("experts_out", (T * top, d), torch.float32)
+        idx = ctx.buffer("router_choice", (T, per), torch.int32)
+        wts = ctx.buffer("router_weights", (T, per), torch.float32)
+        offsets = ctx.buffer("router_runs", (E + more + 1,), torch.int32)
+        pairs = ctx.buffer("router_pairs", (T * per,), torch.int32)
+        K.route(logits, top, idx, wts, offsets, pairs, always=self.merged)
+        hidden = ctx.buffer("experts_hidden", (T * per, F), self.dtype)
+        K.expert_gemm(h, self.w_up, hidden, act=self.act, offsets=offsets, pairs=pairs, a_div=per, mfma=mfma)
+        outs = ctx.buffer("experts_out", (T * per, d), torch.float32)
         K.expert_gemm(hidden, self.w_down, outs, offsets=offsets, pairs=pairs, mfma=mfma)
         if epilogue == ops.EPI_ADD:
             ops.settle_residual(ctx, x)
         first = epilogue == ops.EPI_STORE          # whether x still has to be written rather than added to
-        if self.shared is not None:
+        if self.shared is not None and not self.merged:
             s_hidden = ctx.buffer("shared_hidden", (T, self.shared.intermediate), self.dtype)
             K.expert_gemm(h, self.s_up, s_hidden, act=self.shared.activation, mfma=mfma)
             if first:

@@ -489,6 +489,22 @@ def test_router_choice_ties_weights_and_runs():
         assert offsets[0] == 0 and offsets[-1] == T * top and sorted(pairs) == list(range(T * top))
         for e in range(E):
             assert all(idx.reshape(-1)[p] == e for p in pairs[offsets[e]:offsets[e + 1]])
+    # one more expert that every token passes, with weight 1, behind a token's choices: in a small step (one launch) and
+    # in a larger one
+    for n, top in ((70, 2), (9, 3), (1, 1)):
+        per = top + 1
+        idx, wts = torch.zeros(n, per, dtype=torch.int32, device=DEV), torch.zeros(n, per, device=DEV)
+        offsets, pairs = torch.zeros(E + 2, dtype=torch.int32, device=DEV), torch.zeros(n * per, dtype=torch.int32, device=DEV)
+        K.route(dev(logits[:n]), top, idx, wts, offsets, pairs, always=True)
+        idx, wts, offsets, pairs = idx.cpu().numpy(), host(wts), offsets.cpu().numpy(), pairs.cpu().numpy()
+        for t in range(n):
+            order = np.argsort(-logits[t], kind="stable")[:top]
+            assert list(idx[t]) == list(order) + [E], (top, t)
+            np.testing.assert_allclose(wts[t], list(P.softmax(logits[t, order].astype(np.float64))) + [1.0], atol=1e-6)
+        assert offsets[0] == 0 and offsets[-1] == n * per and sorted(pairs) == list(range(n * per))
+        assert sorted(pairs[offsets[E]:]) == [t * per + top for t in range(n)]
+        for e in range(E + 1):
+            assert all(idx.reshape(-1)[p] == e for p in pairs[offsets[e]:offsets[e + 1]])
 
 
 @pytest.mark.parametrize("dtype, mfma", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
