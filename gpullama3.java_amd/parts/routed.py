@@ -7,7 +7,9 @@ choice) pairs are ordered by expert on the device, and two grouped products (``l
 belongs to one expert) make the experts' hidden rows and their outputs; the weighted sum runs over a token's pairs
 in the order of its choices. A pair's numbers depend on its token and expert alone, so a token's output does not
 depend on its batch-mates; no expert has a capacity, no token is dropped. Nothing waits for the host: the launches'
-shapes follow from the step's number of tokens, so decode steps can be captured.
+shapes follow from the step's number of tokens, so decode steps can be captured. A shared expert with the experts' own
+sizes and activation is stacked behind them as expert number E, and every token gets one more pair for it with weight
+1: its products and its part of the sum ride in the experts' launches. One of another form has two products of its own.
 """
 from __future__ import annotations
 
