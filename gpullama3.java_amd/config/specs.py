@@ -29,12 +29,24 @@ class LinearRopeScaling:
 
 
 @dataclass(frozen=True)
+class YarnRopeScaling:
+    """Pairs that turn fast keep their frequency, pairs that turn slowly have it divided by ``factor``, with a linear
+    ramp over the pair's number in between: from the (fractional, rounded down) number of the pair whose wave makes
+    ``fast`` turns over ``original_max_position`` positions to the (rounded up) one that makes ``slow`` turns. cos and
+    sin are multiplied by ``0.1 ln(factor) + 1``."""
+    factor: float
+    original_max_position: int
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
 class RotarySpec:
     """Rotary position encoding of queries and keys."""
     kind: str = "rotary"
     head_dim: int = 0
     theta: float = 10000.0
-    scaling: object = None       # None, a Llama3RopeScaling or a LinearRopeScaling
+    scaling: object = None       # None, a Llama3RopeScaling, a LinearRopeScaling or a YarnRopeScaling
     pairing: str = "half"        # "half": (j, j + hs/2); "adjacent": (2j, 2j+1)
     max_positions: int = 0
 
@@ -107,6 +119,9 @@ class AttentionSpec:
                                       # ``k_norm`` (shared by the heads) before the rotation; None: no such norm
     chunk: Optional[int] = None       # n: query i sees key j <= i only if i // n == j // n (chunks count from position 0)
     differential: Optional[Differential] = None
+    values_are_keys: bool = False     # no value projection: a position's values are its keys as projected (before the
+                                      # norm on keys and the rotation); ``names`` then has no ``v``
+    # (a name ``sink`` among ``names``: a stored [n_heads] vector, a learned sink per query head in place of ``sink``)
     # (no ``k`` among ``names``: the mixer has no keys and values of its own and only ever reads another entry's)
     # (a name ``head_gate`` among ``names``: a stored [n_heads, hidden] matrix; head h's output is multiplied by
     # sigmoid of its row's product with the mixer's input, before the output projection)
@@ -156,6 +171,29 @@ class SideBySideSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal attention whose keys and values are expanded from one latent per position (``parts/latent_attention.py``).
+    Queries: ``c_q = RMSnorm(W_dq h)`` (``q_rank`` elements), ``q = W_uq c_q``, per head [``head_dim`` unrotated |
+    ``rot_dim`` rotated]. ``W_dkv h`` gives the latent c (``kv_rank``, RMS-normed) and ``rot_dim`` more elements, one
+    rotated key part for all heads. Per head the unrotated key is ``W_uk c`` and the value ``W_uv c``
+    (``v_head_dim``); score = (q . k over both parts) * ``scale``; an ordinary softmax; the heads' outputs times
+    sigmoid of a gate projection of the mixer's input; output projection. Only c and the rotated part are cached."""
+    kind: str = "latent_attention"
+    hidden: int = 0
+    n_heads: int = 0
+    head_dim: int = 0
+    rot_dim: int = 0
+    v_head_dim: int = 0
+    q_rank: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+    position: Optional[RotarySpec] = None      # over the rot_dim part
+    norm_eps: float = 1e-5
+    names: dict = field(default_factory=dict)  # "dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv", "g", "o"
+    out_mult: float = 1.0
+
+
+@dataclass(frozen=True)
 class RetentionSpec:
     """Linear attention with a fixed decay per head and no softmax (``parts/retention.py``): per head a matrix
     S [key_dim, value_dim] in 32-bit, ``S <- decay_h S + k v^T`` with k times ``key_dim ** -0.5``, ``o = S^T q``; q and
@@ -169,8 +207,14 @@ class RetentionSpec:
     decay: tuple = ()                 # one factor per head
     position: Optional[RotarySpec] = None
     norm_eps: float = 1e-5
-    names: dict = field(default_factory=dict)     # "q", "k", "v", "g", "o"
+    names: dict = field(default_factory=dict)     # "q", "k", "v", "g", "o" (and "norm", see ``norm_over``)
     out_mult: float = 1.0
+    # what other linear attentions of this form change:
+    key_scale: Optional[float] = None     # the factor on k; None: key_dim ** -0.5
+    input_activation: Optional[str] = None    # "silu": q, k and v pass silu behind their projections
+    norm_over: str = "head"               # "head": each head's read-out divided by its root mean square; "all": the heads'
+                                          # read-outs together, times the stored weight ``norm`` [n_heads value_dim]
+    gate_activation: str = "silu"         # "silu" or "sigmoid" of the gate projection
 
 
 @dataclass(frozen=True)
@@ -229,10 +273,14 @@ class GatedFeedForwardSpec:
 
 @dataclass(frozen=True)
 class ExpertSpec:
-    """One small feed-forward without a gate: ``down(act(up h))``; ``activation`` "gelu" (the erf form), "gelu_tanh"
-    or "silu"."""
+    """One small feed-forward. Without a gate: ``down(act(up h))``; ``activation`` "gelu" (the erf form), "gelu_tanh"
+    or "silu". ``gated``: ``down(act(min(gate h, limit)) * (clamp(up h, -limit, limit) + up_shift))`` with
+    ``activation`` one of the gated feed-forward's ("silu", "gelu_tanh", "quick_gelu"); ``limit`` None: unbounded."""
     intermediate: int = 0
     activation: str = "gelu"
+    gated: bool = False
+    limit: Optional[float] = None
+    up_shift: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -249,6 +297,14 @@ class RoutedFeedForwardSpec:
     shared: Optional[ExpertSpec] = None
     names: dict = field(default_factory=dict)
     out_mult: float = 1.0
+    # Another rule for the choice (``weights = "scores"``): s = softmax of the router's outputs over ALL experts; the
+    # ``top`` largest of s + the stored ``correction`` are chosen; their weights are their s divided by the chosen s'
+    # sum plus ``sum_eps``. "chosen_softmax": the softmax over the chosen logits alone.
+    weights: str = "chosen_softmax"
+    sum_eps: float = 0.0
+    n_identity: int = 0               # the router's last outputs stand for experts whose output is their input (no tensors);
+                                      # the router has n_experts + n_identity rows
+    # (names: ``expert_gate`` beside ``expert_up`` / ``expert_down`` for gated experts, ``shared_gate``; ``correction``)
 
 
 @dataclass(frozen=True)
@@ -256,12 +312,17 @@ class BlockSpec:
     """One layer: how norm, mixer and feed-forward are arranged is ``kind``. "prenorm": x += mixer(norm(x));
     x += ffn(norm(x)). "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h) (one norm, ``ffn_norm`` is None).
     "outnorm": x += mixer_norm(mixer(x)); x += ffn_norm(ffn(x)): the sublayers read the rows themselves, the norms
-    stand behind them."""
+    stand behind them. "streams": every token has ``ModelSpec.streams`` copies x_1 .. x_S of its row; a sublayer reads
+    norm(sum_s in[s] x_s) and its output y goes back as x_r <- sum_s mix[s, r] x_s + out[r] y (all r at once); the
+    numbers are stored per sublayer under ``stream_names`` ("mixer_in" [S], "mixer_mix" [S, S], "mixer_out" [S], and
+    the same with "ffn_")."""
     kind: str = "prenorm"
     mixer_norm: object = None
     mixer: object = None
     ffn_norm: object = None
     ffn: object = None
+    streams: int = 1
+    stream_names: dict = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -328,3 +389,5 @@ class ModelSpec:
     logit_softcap: Optional[float] = None         # the logits become cap * tanh(logits / cap) (after the scale)
     unused_tensor_names: tuple = ()               # stored names that a folder may hold although nothing reads them
     pair_embedding: Optional[PairEmbedding] = None   # a row per (previous token, token) added to the embedding's output
+    streams: int = 1                              # copies of the residual row per token (blocks of kind "streams"); all
+                                                  # start as the embedding's output, and their sum goes to the final norm

@@ -63,7 +63,8 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits,
-    const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
+    const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps,
+    const float* __restrict__ sinks) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
   constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
@@ -234,6 +235,10 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   float M = sm_m[0][j];
 #pragma unroll
   for (int w = 1; w < NS; ++w) M = fmaxf(M, sm_m[w][j]);
+  if (BIAS && sinks) {                          // a sink per query head (a lane beyond the group's heads reads the last head's)
+    has_sink = 1;
+    sink = sinks[min(h0 + j * hstep, n_heads - 1)];
+  }
   const bool sink_here = BIAS && has_sink && n_splits == 1;
   if (sink_here) M = fmaxf(M, sink);
   float f[NS], L = sink_here ? __expf(sink - M) : 0.f;
@@ -272,9 +277,14 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
 __global__ __launch_bounds__(64) void attention_decode_merge_kernel(const float* __restrict__ part_o,
                                                                     const float* __restrict__ part_ml,
                                                                     bf16_t* __restrict__ out, long out_stride, int n_heads,
-                                                                    int head_dim, int n_splits, int has_sink, float sink) {
+                                                                    int head_dim, int n_splits, int has_sink, float sink,
+                                                                    const float* __restrict__ sinks) {
   const long th = blockIdx.x;   // token * n_heads + head
   const long t = th / n_heads, h = th % n_heads;
+  if (sinks) {
+    has_sink = 1;
+    sink = sinks[h];
+  }
   const int lane = threadIdx.x;
   const float* ml = part_ml + th * n_splits * 2;
   float m[4], l[4];             // (at most 256 splits)
@@ -327,7 +337,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                                     int table_stride, float* part_o, float* part_ml, long part_floats, void* out,
                                     long out_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
                                     int window, float scale, int n_splits, const float* slopes, int has_sink, float sink,
-                                    int keep_first, int mask_chunk, int maps, hipStream_t stream) {
+                                    int keep_first, int mask_chunk, int maps, const float* sinks, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && block_table && out && table_stride > 0,
               "gl3_attention_decode: null argument");
@@ -356,11 +366,11 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   // first to end (what a block does before its keys arrive is a chain of trips to memory, paid once per round).
   const bool small = blocks * n_splits > 256;
   GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_decode: %d kept first keys without a window", keep_first);
-  const bool biased = slopes != nullptr || has_sink || keep_first > 0;    // (the kernels that know of kept first keys)
+  const bool biased = slopes != nullptr || has_sink || sinks != nullptr || keep_first > 0;    // (the kernels that know of kept first keys)
 #define AD_ARGS                                                                                                       \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table,    \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, n_heads / n_kv, page_size, page_shift, window,  \
-      scale, n_splits, slopes, has_sink, sink, keep_first, mask_chunk, maps
+      scale, n_splits, slopes, has_sink, sink, keep_first, mask_chunk, maps, sinks
 #define GO(HS)                                                                                                        \
   do {                                                                                                                \
     constexpr int CB = HS <= 64 ? 4 : HS <= 96 ? 3 : 2;                                                               \
@@ -386,7 +396,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   GL3_LAUNCH_CHECK();
   if (n_splits > 1) {
     attention_decode_merge_kernel<<<dim3((unsigned)((long)n_tokens * n_heads)), dim3(64), 0, stream>>>(
-        part_o, part_ml, (bf16_t*)out, out_stride, n_heads, head_dim, n_splits, has_sink, sink);
+        part_o, part_ml, (bf16_t*)out, out_stride, n_heads, head_dim, n_splits, has_sink, sink, sinks);
     GL3_LAUNCH_CHECK();
   }
   return 0;

@@ -20,19 +20,21 @@
 // window): query p sees key j <= p only if j / chunk == p / chunk. And fewer value heads than key heads (n_v): several
 // score maps over the same values. With maps = n_kv / n_v, query heads and key heads lie head by head as [map 0, map 1,
 // ...]: query head h is map h % maps of head h / maps, which reads key head g * maps + h % maps and value head g, g the
-// head's group.
+// head's group. The sink may be a number per query head (sinks). And values that are a part of the keys (v_in_k >= 0): a
+// cache with one array per position, whose elements v_in_k .. v_in_k + v_head_dim are the values (an attention over
+// cached latents); heads of up to 1024 elements then (MAXHS 1024: more registers, so a kernel of its own).
 #include "common.h"
 
 #define ATT_MAX_HS 256
 
-template <typename T, typename TO>
+template <typename T, typename TO, int MAXHS>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, TO* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
     int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink, int keep_first,
-    int chunk, int n_v) {
-  __shared__ float qs[ATT_MAX_HS];
+    int chunk, int n_v, const float* __restrict__ sinks, int v_in_k) {
+  __shared__ float qs[MAXHS];
   __shared__ float ps[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = positions[t];
@@ -45,8 +47,12 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   for (int i = lane; i < head_dim; i += 64) qs[i] = to_f32<T>(qp[i]);
   __syncthreads();
   const float slope = slopes ? slopes[h] : 0.f;
+  if (sinks) {
+    has_sink = 1;
+    sink = sinks[h];
+  }
   float m = has_sink ? sink : -INFINITY, l = has_sink ? 1.f : 0.f;
-  float acc[ATT_MAX_HS / 64] = {};
+  float acc[MAXHS / 64] = {};
   // with a window, the sequence's first keep_first keys stay visible: those of them that lie before the window are
   // visited first, in chunks of their own, then the window's keys
   const int kept = keep_first < lo ? keep_first : lo;
@@ -72,15 +78,25 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     __syncthreads();
     const int n_valid = (to - base + 1 < 64) ? to - base + 1 : 64;
 #pragma unroll
-    for (int r = 0; r < ATT_MAX_HS / 64; ++r) acc[r] *= alpha;
+    for (int r = 0; r < MAXHS / 64; ++r) acc[r] *= alpha;
     for (int j = 0; j < n_valid; ++j) {
       const int kj = base + j;
-      // values lie transposed in a page: [head_dim][position in page], in tiles
-      const T* vp = v_cache + ((long)bt[kj / page_size] * n_v + cv) * page_size * v_head_dim;
       const int in_page = kj % page_size;
       const float w = ps[j];
+      if (v_in_k >= 0) {
+        // the values are elements of the key rows themselves
+        const T* kp = k_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * head_dim;
 #pragma unroll
-      for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
+        for (int r = 0; r < MAXHS / 64; ++r) {
+          const int i = lane + 64 * r;
+          if (i < v_head_dim) acc[r] = fmaf(w, to_f32<T>(kp[gl3_k_offset(in_page, v_in_k + i, head_dim)]), acc[r]);
+        }
+        continue;
+      }
+      // values lie transposed in a page: [head_dim][position in page], in tiles
+      const T* vp = v_cache + ((long)bt[kj / page_size] * n_v + cv) * page_size * v_head_dim;
+#pragma unroll
+      for (int r = 0; r < MAXHS / 64; ++r) {
         const int i = lane + 64 * r;
         if (i < v_head_dim) acc[r] = fmaf(w, to_f32<T>(vp[gl3_v_offset(i, in_page, page_size)]), acc[r]);
       }
@@ -90,7 +106,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   }
   TO* op = out + (long)t * out_stride + (long)h * v_head_dim;
 #pragma unroll
-  for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
+  for (int r = 0; r < MAXHS / 64; ++r) {
     const int i = lane + 64 * r;
     if (i < v_head_dim) op[i] = from_f32<TO>(acc[r] / l);
   }
@@ -101,16 +117,18 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
                                      int table_stride, void* out, long out_stride, int n_tokens, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int v_head_dim,
                                      const float* slopes, int has_sink, float sink, int keep_first, int chunk, int n_v,
-                                     int out_dtype, hipStream_t stream) {
+                                     int out_dtype, const float* sinks, int v_in_k, hipStream_t stream) {
   if (n_tokens == 0) return 0;
-  GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
+  GL3_REQUIRE(q && k_cache && (v_cache || v_in_k >= 0) && positions && seq_of_token && block_table && out,
               "gl3_attention_generic: null argument");
   GL3_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
               "gl3_attention_generic: %d heads over %d kv heads", n_heads, n_kv);
-  GL3_REQUIRE(head_dim > 0 && head_dim <= ATT_MAX_HS, "gl3_attention_generic: head_dim %d exceeds %d", head_dim,
-              ATT_MAX_HS);
-  GL3_REQUIRE(v_head_dim > 0 && v_head_dim <= ATT_MAX_HS && v_head_dim % 16 == 0,
-              "gl3_attention_generic: v_head_dim %d is not a multiple of 16 up to %d", v_head_dim, ATT_MAX_HS);
+  const int most = v_in_k >= 0 ? 1024 : ATT_MAX_HS;
+  GL3_REQUIRE(head_dim > 0 && head_dim <= most, "gl3_attention_generic: head_dim %d exceeds %d", head_dim, most);
+  GL3_REQUIRE(v_head_dim > 0 && v_head_dim <= most && (v_head_dim % 16 == 0 || v_in_k >= 0),
+              "gl3_attention_generic: v_head_dim %d is not a multiple of 16 up to %d", v_head_dim, most);
+  GL3_REQUIRE(v_in_k < 0 || (v_in_k + v_head_dim <= head_dim && n_v == n_kv),
+              "gl3_attention_generic: values of %d from element %d of keys of %d", v_head_dim, v_in_k, head_dim);
   GL3_REQUIRE(n_heads <= 65535, "gl3_attention_generic: %d heads exceed the grid", n_heads);
   GL3_REQUIRE(page_size > 0 && table_stride > 0, "gl3_attention_generic: bad paging");
   GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_generic: %d kept first keys without a window", keep_first);
@@ -121,17 +139,23 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
               "gl3_attention_generic: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16", page_size,
               head_dim);
   dim3 grid(n_tokens, n_heads), block(64);
-#define ATT_GENERIC(T, TO)                                                                                             \
-  attention_generic_kernel<T, TO><<<grid, block, 0, stream>>>(                                                         \
+#define ATT_GENERIC_OF(T, TO, MAXHS)                                                                                   \
+  attention_generic_kernel<T, TO, MAXHS><<<grid, block, 0, stream>>>(                                                  \
       (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, positions, seq_of_token, block_table, table_stride, \
       (TO*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink, sink,     \
-      keep_first, chunk, n_v)
+      keep_first, chunk, n_v, sinks, v_in_k)
+#define ATT_GENERIC(T, TO)                                                       \
+  do {                                                                           \
+    if (head_dim <= ATT_MAX_HS && v_head_dim <= ATT_MAX_HS) ATT_GENERIC_OF(T, TO, ATT_MAX_HS); \
+    else ATT_GENERIC_OF(T, TO, 1024);                                            \
+  } while (0)
   // (the output in 32-bit beside 16-bit operands: for a caller that goes on in 32-bit with the heads' outputs)
   if (dtype == GL3_F32 && out_dtype == GL3_F32) ATT_GENERIC(float, float);
   else if (dtype == GL3_BF16 && out_dtype == GL3_BF16) ATT_GENERIC(bf16_t, bf16_t);
   else if (dtype == GL3_BF16 && out_dtype == GL3_F32) ATT_GENERIC(bf16_t, float);
   else GL3_REQUIRE(false, "gl3_attention_generic: dtypes %d -> %d are not built", dtype, out_dtype);
 #undef ATT_GENERIC
+#undef ATT_GENERIC_OF
   GL3_LAUNCH_CHECK();
   return 0;
 }

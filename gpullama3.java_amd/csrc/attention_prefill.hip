@@ -46,7 +46,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps,
+    const float* __restrict__ sinks) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
   constexpr int KROW = HS + 8;            // a key row in shared memory, in elements
@@ -115,8 +116,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   for (int hh = 0; hh < GH; ++hh) {
     m_run[hh] = -INFINITY;
     l_run[hh] = 0.f;
-    if (BIAS && has_sink) {                     // (a lane holds its quarter's share of the row sum: the sink's 1 once a query)
-      m_run[hh] = sink * 1.4426950408889634f;
+    if (BIAS && (has_sink || sinks)) {          // (a lane holds its quarter's share of the row sum: the sink's 1 once a query)
+      m_run[hh] = (sinks ? sinks[min(head_at(hh), n_heads - 1)] : sink) * 1.4426950408889634f;
       l_run[hh] = qd == 0 ? 1.f : 0.f;
     }
 #pragma unroll
@@ -294,7 +295,8 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first, int mask_chunk, int maps,
+    const float* __restrict__ sinks) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
   constexpr int NT = CK / 32;             // score tiles of a chunk of CK keys
@@ -347,8 +349,8 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     qt[kk] = q_ok ? *(const bf16x8*)(q + (long)(tok0 + qi0 + n) * q_stride + (long)head * HS + kk * 16 + 8 * h) : zero8;
 
   float m_run = -INFINITY, l_run = 0.f;
-  if (BIAS && has_sink) {                       // (two lanes share a query's row sum: the sink's 1 once)
-    m_run = sink * 1.4426950408889634f;
+  if (BIAS && (has_sink || sinks)) {            // (two lanes share a query's row sum: the sink's 1 once)
+    m_run = (sinks ? sinks[head] : sink) * 1.4426950408889634f;
     l_run = h == 0 ? 1.f : 0.f;
   }
   const float sl = (BIAS && slopes) ? slopes[head] / scale : 0.f;
@@ -538,7 +540,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
                                      const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
                                      int max_q_len, int n_heads, int n_kv, int head_dim, int page_size, int window,
                                      float scale, int wide_from, const float* slopes, int has_sink, float sink,
-                                     int keep_first, int mask_chunk, int maps, hipStream_t stream) {
+                                     int keep_first, int mask_chunk, int maps, const float* sinks, hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && cu_seqlens && kv_before && block_table && out,
               "gl3_attention_prefill: null argument");
@@ -564,11 +566,11 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
               n_seqs, q_blocks);
   dim3 grid((unsigned)z, n_seqs, q_blocks), block(256);
   GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_prefill: %d kept first keys without a window", keep_first);
-  const bool biased = slopes != nullptr || has_sink || keep_first > 0;    // (the kernels that know of kept first keys)
+  const bool biased = slopes != nullptr || has_sink || sinks != nullptr || keep_first > 0;    // (the kernels that know of kept first keys)
   if (wide) {
 #define PF_ARGS                                                                                                     \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table,     \
-      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink, keep_first, mask_chunk, maps
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink, keep_first, mask_chunk, maps, sinks
 #define GOW(HS, CK, AH, OCC)                                                                                        \
   do {                                                                                                              \
     if (biased) attention_prefill_wide_kernel<HS, CK, AH, OCC, true><<<grid, block, 0, stream>>>(PF_ARGS);          \

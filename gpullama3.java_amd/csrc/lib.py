@@ -57,7 +57,7 @@ def _declare(lib):
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, F, F, P, P],
-        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, I, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, I, P, I, P],
         "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
         "gl3_concat_rows": [P, P, P, I, I, I, P],
         "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P, P, F, P],
@@ -66,11 +66,17 @@ def _declare(lib):
         "gl3_layernorm_add": [P, P, P, P, I, I, F, P, I, P],
         "gl3_cast_rows": [P, P, I, L, P],
         "gl3_ssm_prep": [P, L, I, I, I, I, I, I, P, P, I, P, P, P, L, L, P, P, P, P, P, P],
-        "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P, L, I, I, P],
-        "gl3_group_norm_gate": [P, P, L, I, P, I, P, L, I, P, F, I, I, I, I, P, I, P],
-        "gl3_route": [P, I, I, I, P, P, P, P, I, P],
-        "gl3_expert_gemm": [P, I, L, I, P, I, I, I, I, P, P, I, P, I, L, I, I, P],
-        "gl3_route_combine": [P, P, I, I, I, P, I, P],
+        "gl3_decay_scan": [P, L, I, P, L, I, P, L, I, P, P, L, P, F, P, L, L, P, P, P, L, I, I, I, I, I, P, L, I, I, I, P],
+        "gl3_group_norm_gate": [P, P, L, I, P, I, P, L, I, P, F, I, I, I, I, P, I, I, P],
+        "gl3_route": [P, I, I, I, P, P, P, P, I, I, P, F, P],
+        "gl3_expert_gemm": [P, I, L, I, P, I, I, I, I, P, P, I, P, I, L, I, I, I, F, F, P],
+        "gl3_route_combine": [P, P, I, I, I, P, I, P, I, P, I, P],
+        "gl3_streams_step": [P, I, I, I, P, P, P, P, P, F, P, I, P],
+        "gl3_streams_fill": [P, P, I, I, I, P],
+        "gl3_streams_sum": [P, P, I, I, I, P, P],
+        "gl3_latent_prep": [P, L, I, I, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, I, I, I, P, P, P],
+        "gl3_latent_query": [P, I, I, I, I, I, P, P, P, P, I, I, P],
+        "gl3_sigmoid_gate": [P, I, P, L, I, I, I, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
@@ -96,13 +102,13 @@ def _declare(lib):
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P, F, F, P, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
-        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
+        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P, P],
         "gl3_scatter_i32": [P, L, P, P, I, P],
         "gl3_upload": [P, P, L, P],
         "gl3_stage_decode": [P, I, I, P, P, P, I, P, P],
         "gl3_stage_step": [P, P, P, I, P, P, P, I, P, I, I, P],
         "gl3_graph_launch": [P, P],
-        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P],
+        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P, I, F, I, I, I, P, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name, None)
@@ -233,6 +239,19 @@ def _slopes(slopes, n_heads, who):
         if slopes.shape != (n_heads,):
             raise KernelError(f"{who}: {tuple(slopes.shape)} slopes for {n_heads} heads")
     return _ptr(slopes)
+
+
+def _sink(sink, n_heads, who):
+    """A sink as the kernels take it: ``(has one number, that number, pointer to one number per head)``. ``sink`` is
+    None, a number, or a float32 tensor [n_heads] on the device."""
+    if sink is None:
+        return 0, 0.0, None
+    if isinstance(sink, torch.Tensor):
+        _dev(sink, "sink", torch.float32)
+        if sink.shape != (n_heads,):
+            raise KernelError(f"{who}: {tuple(sink.shape)} sinks for {n_heads} heads")
+        return 0, 0.0, _ptr(sink)
+    return 1, float(sink), None
 
 
 def _act(act, who):
@@ -400,8 +419,11 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu", act_limit
 
 
 def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None, keep_first=0, chunk=0, n_v_heads=None):
-    """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries. ``v_head_dim``: the values'
+                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None, keep_first=0, chunk=0, n_v_heads=None,
+                      values_in_keys=None):
+    """``sink`` may also be a float32 tensor [H]: a sink per query head. ``values_in_keys``: n: the cache has no value
+    array (``v_cache`` None); the values are elements n .. n + v_head_dim of the key rows (heads of up to 1024).
+    q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries. ``v_head_dim``: the values'
     size where it is not the keys'; ``slopes``: float32 [H], score - slopes[h] * distance; ``sink``: the score of a
     key without a value that every query sees (None: no such key); ``keep_first``: with a window, the sequence's
     first keys that stay visible to every later query; ``chunk``: n > 0: query i sees key j <= i only if
@@ -409,7 +431,11 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     score maps over the same values, ``maps = n_kv / n_v_heads``; query and key heads then lie head by head as
     [map 0, map 1, ...], and map m of a head reads key head ``g * maps + m`` and value head g of the head's group."""
     _dev(q, "q", contiguous=False); _dev(out, "out", contiguous=False)
-    _dev(k_cache, "k_cache", q.dtype); _dev(v_cache, "v_cache", q.dtype)
+    _dev(k_cache, "k_cache", q.dtype)
+    if values_in_keys is None:
+        _dev(v_cache, "v_cache", q.dtype)
+    elif v_cache is not None or n_v_heads is not None:
+        raise KernelError("attention: values inside the keys come without a value array and with as many value heads")
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
     _dev(block_table, "block_table", torch.int32)
     T = q.shape[0]
@@ -419,9 +445,15 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     if out.shape != (T, n_heads * vd) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
     n_v = n_kv if n_v_heads is None else int(n_v_heads)
-    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", vd, n_v)
+    if values_in_keys is None:
+        _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", vd, n_v)
+    elif (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or values_in_keys < 0
+          or values_in_keys + vd > head_dim):
+        raise KernelError(f"attention: keys {tuple(k_cache.shape)} for {n_kv} heads of {head_dim} in pages of {page_size}, "
+                          f"values of {vd} from element {values_in_keys}")
     if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
+    has_sink, sink_value, sinks = _sink(sink, n_heads, "attention")
     if chunk and window:
         raise KernelError("attention: a chunked mask has no window")
     if slopes is not None:
@@ -431,8 +463,9 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     _check(library().gl3_attention_generic(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
-        int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0),
-        int(keep_first or 0) if window else 0, int(chunk or 0), n_v, _code(out, "out"), _stream()),
+        int(window or 0), float(scale), vd, _ptr(slopes), has_sink, sink_value,
+        int(keep_first or 0) if window else 0, int(chunk or 0), n_v, _code(out, "out"), sinks,
+        -1 if values_in_keys is None else int(values_in_keys), _stream()),
         "attention_generic")
 
 
@@ -667,13 +700,14 @@ def scan_pieces_floats(max_len, n_seqs, H, N, P):
 
 
 def decay_scan(q, col_q, k, col_k, v, col_v, state, state_off, cu_seqlens, slot_ids, out, H, heads_per_group, N, P,
-               a_tok=None, b_tok=None, a_head=None, b_const=1.0, pieces=None, max_len=0):
+               a_tok=None, b_tok=None, a_head=None, b_const=1.0, pieces=None, max_len=0, silu_inputs=False):
     """Per (sequence, head) ``S <- a S + b k v^T`` and ``o = S^T q`` token by token, S [N, P] float32 in ``state``
     [slots, *] from ``state_off + h N P`` on. q and k: float32 rows whose group g (``heads_per_group`` heads share one)
     starts at column ``col + g N``; v: head h at ``col_v + h P``. a and b: per token and head (``a_tok``, ``b_tok``,
     columns h of rows of the same stride) or per head (``a_head`` [H]) / one number (``b_const``). ``out`` [T, H P].
     With ``pieces`` (float32 scratch of ``scan_pieces_floats`` elements) and ``max_len`` (the longest sequence of the
-    step) a long step runs as pieces side by side, joined through their start states."""
+    step) a long step runs as pieces side by side, joined through their start states. ``silu_inputs``: q, k and v pass
+    silu as they are read."""
     groups = H // heads_per_group
     _f32_rows(q, "q", col_q + groups * N); _f32_rows(k, "k", col_k + groups * N); _f32_rows(v, "v", col_v + H * P)
     _dev(out, "out", torch.float32)
@@ -705,13 +739,16 @@ def decay_scan(q, col_q, k, col_k, v, col_v, state, state_off, cu_seqlens, slot_
                                     state.stride(0), int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
                                     out.stride(0), B, int(H), int(heads_per_group), int(N), int(P),
                                     _ptr(pieces) if piece_len else None, pieces.numel() if piece_len else 0, int(max_len),
-                                    int(piece_len), _stream()), "decay_scan")
+                                    int(piece_len), int(bool(silu_inputs)), _stream()), "decay_scan")
 
 
-def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=False, skip=None):
+def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=False, skip=None, gate_act="silu"):
     """``o`` [T, C] float32 (+ ``skip = (rows, col, d [heads], head_dim)``: d[h] times the rows' columns), times silu of
     the gate columns (``gate`` rows float32 from ``col_g``) before (``gate_first``) or after being divided by its root
-    mean square over every ``gsize`` channels; times ``weight`` [C]. ``out`` [T, C] in the activations' type."""
+    mean square over every ``gsize`` channels; times ``weight`` [C]. ``out`` [T, C] in the activations' type.
+    ``gate_act``: "silu" or "sigmoid" of the gate columns."""
+    if gate_act not in ("silu", "sigmoid"):
+        raise KernelError(f"group_norm_gate: a gate's {gate_act!r} is not built (silu, sigmoid)")
     _dev(o, "o", torch.float32); _dev(out, "out")
     T, C = o.shape
     _f32_rows(gate, "gate", col_g + C)
@@ -731,21 +768,26 @@ def group_norm_gate(o, gate, col_g, out, gsize, eps, weight=None, gate_first=Fal
         ld_x = sx.stride(0)
     _check(library().gl3_group_norm_gate(_ptr(o), _ptr(sx), ld_x, int(col_x), _ptr(sd), int(hd), _ptr(gate), gate.stride(0),
                                          int(col_g), _ptr(weight), float(eps), int(bool(gate_first)), T, C, int(gsize),
-                                         _ptr(out), _code(out, "out"), _stream()), "group_norm_gate")
+                                         _ptr(out), _code(out, "out"), int(gate_act == "sigmoid"), _stream()), "group_norm_gate")
 
 
 EXPERT_ACTIVATIONS = {None: 0, "gelu": 1, "gelu_tanh": 2, "silu": 3}
 ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS = 16, 1024      # as csrc/routed.hip has them
 
 
-def route(logits, top, idx, wts, offsets, pairs, always=False):
+def route(logits, top, idx, wts, offsets, pairs, always=False, scores=False, correction=None, sum_eps=0.0):
     """Router logits [T, E] float32 -> the ``top`` largest per token (``idx`` [T, top] int32, the lower number wins a
     tie) with the softmax over them alone (``wts`` [T, top]); and the (token, choice) pairs ordered by expert:
     ``offsets`` [E + 1] int32, ``pairs`` [T top] int32 (pair t * top + j). ``always``: every token has one more pair
     behind its choices, with expert number E and weight 1 (``idx`` and ``wts`` [T, top + 1], ``offsets`` [E + 2],
-    ``pairs`` [T (top + 1)])."""
+    ``pairs`` [T (top + 1)]). ``scores``: the other rule: s = softmax over all E logits, the choice goes by
+    s + ``correction`` (float32 [E], optional), the weights are the chosen s divided by their sum plus ``sum_eps``."""
     _dev(logits, "logits", torch.float32)
     T, E = logits.shape
+    if correction is not None:
+        _dev(correction, "correction", torch.float32)
+        if not scores or correction.shape != (E,):
+            raise KernelError(f"route: a correction {tuple(correction.shape)} for {E} scores")
     more = 1 if always else 0
     for t, name, shape, dt in ((idx, "idx", (T, top + more), torch.int32), (wts, "wts", (T, top + more), torch.float32),
                                (offsets, "offsets", (E + more + 1,), torch.int32),
@@ -754,21 +796,30 @@ def route(logits, top, idx, wts, offsets, pairs, always=False):
         if tuple(t.shape) != shape:
             raise KernelError(f"route: {name} {tuple(t.shape)}, expected {shape}")
     _check(library().gl3_route(_ptr(logits), T, E, int(top), _ptr(idx), _ptr(wts), _ptr(offsets), _ptr(pairs),
-                               E if always else -1, _stream()), "route")
+                               E if always else -1, int(bool(scores)), _ptr(correction), float(sum_eps), _stream()), "route")
 
 
-def expert_gemm(a, w, out, act=None, offsets=None, pairs=None, a_div=1, mfma=True):
+def expert_gemm(a, w, out, act=None, offsets=None, pairs=None, a_div=1, mfma=True, gated=None):
     """``out[p] = act(w[e] @ a[p // a_div])`` for every pair p of expert e's run (``offsets``, ``pairs`` of ``route``);
     without them ``w`` is one expert [1, N, K] that takes every row of ``a`` in its own order. ``w`` [E, N, K];
-    ``out`` [pairs, N] in bfloat16 or float32."""
+    ``out`` [pairs, N] in bfloat16 or float32. ``gated = (activation, limit, shift)``: the rows of every ``w[e]`` are
+    gate and up rows in turns (2n: gate n, 2n + 1: up n) and ``out`` [pairs, N / 2] = act(min(gate, limit)) *
+    (clamp(up, -limit, limit) + shift) (``limit`` None or 0: unbounded); ``act`` is then None. ``offsets`` may run on
+    behind the E experts of ``w`` (experts without a product of their own): their pairs are left alone."""
     _dev(a, "a", contiguous=False); _dev(w, "w", a.dtype); _dev(out, "out", contiguous=False)
-    if w.dim() != 3 or a.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1 or a.shape[1] != w.shape[2] or out.shape[1] != w.shape[1]:
+    n_out = w.shape[1] // 2 if gated is not None and w.dim() == 3 else (w.shape[1] if w.dim() == 3 else -1)
+    if w.dim() != 3 or a.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1 or a.shape[1] != w.shape[2] or out.shape[1] != n_out:
         raise KernelError(f"expert_gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
     E, N, K = w.shape
     n_rows = out.shape[0]
+    gate_act, limit, shift = -1, 0.0, 0.0
+    if gated is not None:
+        if act is not None or gated[0] not in ACTIVATIONS or N % 2:
+            raise KernelError(f"expert_gemm: a gated product of {N} rows with {gated[0]!r} ({sorted(ACTIVATIONS)}), act {act!r}")
+        gate_act, limit, shift = ACTIVATIONS[gated[0]], float(gated[1] or 0.0), float(gated[2])
     if offsets is not None:
         _dev(offsets, "offsets", torch.int32); _dev(pairs, "pairs", torch.int32)
-        if offsets.numel() != E + 1 or pairs.numel() != n_rows or a.shape[0] * a_div < n_rows:
+        if offsets.numel() < E + 1 or pairs.numel() != n_rows or a.shape[0] * a_div < n_rows:
             raise KernelError(f"expert_gemm: {offsets.numel()} offsets, {pairs.numel()} pairs, {a.shape[0]} rows x {a_div}")
     elif E != 1 or a.shape[0] != n_rows or a_div != 1:
         raise KernelError("expert_gemm: without runs one expert takes every row")
@@ -776,17 +827,127 @@ def expert_gemm(a, w, out, act=None, offsets=None, pairs=None, a_div=1, mfma=Tru
         raise KernelError(f"expert_gemm: activation {act!r} is not built ({sorted(k for k in EXPERT_ACTIVATIONS if k)})")
     _check(library().gl3_expert_gemm(_ptr(a), _code(a, "a"), a.stride(0), int(a_div), _ptr(w), _code(w, "w"), E, N, K,
                                      _ptr(offsets), _ptr(pairs), n_rows, _ptr(out), _code(out, "out"), out.stride(0),
-                                     EXPERT_ACTIVATIONS[act], int(bool(mfma)), _stream()), "expert_gemm")
+                                     EXPERT_ACTIVATIONS[act], int(bool(mfma)), gate_act, limit, shift, _stream()), "expert_gemm")
 
 
-def route_combine(y, wts, out, accumulate=False):
-    """``out[t]`` (+)= sum over j of ``wts[t, j] * y[t * top + j]``; y [T top, d] float32, out [T, d] float32."""
+def route_combine(y, wts, out, accumulate=False, identity=None):
+    """``out[t]`` (+)= sum over j of ``wts[t, j] * y[t * top + j]``; y [T top, d] float32, out [T, d] float32.
+    ``identity = (idx [T, top] int32, n_real, h [T, d])``: a pair whose expert number is ``n_real`` or more stands for
+    the token's input row ``h[t]`` itself."""
     _dev(y, "y", torch.float32); _dev(wts, "wts", torch.float32); _dev(out, "out", torch.float32)
     T, top = wts.shape
     if y.dim() != 2 or y.shape[0] != T * top or out.shape != (T, y.shape[1]):
         raise KernelError(f"route_combine: y {tuple(y.shape)}, wts {tuple(wts.shape)}, out {tuple(out.shape)}")
-    _check(library().gl3_route_combine(_ptr(y), _ptr(wts), T, top, y.shape[1], _ptr(out), int(bool(accumulate)), _stream()),
+    idx = h = None
+    n_real = 0
+    if identity is not None:
+        idx, n_real, h = identity
+        _dev(idx, "idx", torch.int32); _dev(h, "h")
+        if idx.shape != wts.shape or h.shape != out.shape:
+            raise KernelError(f"route_combine: choices {tuple(idx.shape)}, input rows {tuple(h.shape)}")
+    _check(library().gl3_route_combine(_ptr(y), _ptr(wts), T, top, y.shape[1], _ptr(out), int(bool(accumulate)), _ptr(idx),
+                                       int(n_real), _ptr(h), _code(h, "h") if h is not None else 0, _stream()),
            "route_combine")
+
+
+def streams_step(rows, S, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps=0.0, h=None):
+    """``rows`` [T, S d] float32: S copies of every token's residual row. With ``y`` [T, d] (a sublayer's output) the
+    copies become ``x_r <- sum_s mix[s, r] x_s + out_w[r] y``; with ``in_w`` [S] the next sublayer's input
+    ``h = RMSnorm(sum_s in_w[s] x_s) * norm_w`` is made from the (new) copies. All numbers float32 on the device."""
+    _dev(rows, "rows", torch.float32)
+    T, d = rows.shape[0], rows.shape[1] // S
+    if rows.dim() != 2 or rows.shape[1] != S * d:
+        raise KernelError(f"streams_step: rows {tuple(rows.shape)} for {S} copies")
+    if y is not None:
+        _dev(y, "y", torch.float32); _dev(mix, "mix", torch.float32); _dev(out_w, "out_w", torch.float32)
+        if y.shape != (T, d) or mix.shape != (S, S) or out_w.shape != (S,):
+            raise KernelError(f"streams_step: y {tuple(y.shape)}, mix {tuple(mix.shape)}, out {tuple(out_w.shape)}")
+    if in_w is not None:
+        _dev(in_w, "in_w", torch.float32); _dev(norm_w, "norm_w", torch.float32); _dev(h, "h")
+        if in_w.shape != (S,) or norm_w.shape != (d,) or h.shape != (T, d):
+            raise KernelError(f"streams_step: in {tuple(in_w.shape)}, norm {tuple(norm_w.shape)}, h {tuple(h.shape)}")
+    _check(library().gl3_streams_step(_ptr(rows), T, int(S), d, _ptr(y), _ptr(mix), _ptr(out_w), _ptr(in_w), _ptr(norm_w),
+                                      float(eps), _ptr(h), _code(h, "h") if h is not None else 0, _stream()), "streams_step")
+
+
+def streams_fill(src, rows, S):
+    """Every one of the S copies in ``rows`` [T, S d] takes ``src`` [T, d] (float32)."""
+    _dev(src, "src", torch.float32); _dev(rows, "rows", torch.float32)
+    T, d = src.shape
+    if rows.shape != (T, S * d):
+        raise KernelError(f"streams_fill: {tuple(src.shape)} into {tuple(rows.shape)} as {S} copies")
+    _check(library().gl3_streams_fill(_ptr(src), _ptr(rows), T, int(S), d, _stream()), "streams_fill")
+
+
+def streams_sum(rows, S, out, which=None):
+    """``out[r]`` = the sum of the S copies of token ``which[r]`` (None: token r); float32."""
+    _dev(rows, "rows", torch.float32); _dev(out, "out", torch.float32)
+    n, d = out.shape
+    if rows.dim() != 2 or rows.shape[1] != S * d:
+        raise KernelError(f"streams_sum: rows {tuple(rows.shape)} as {S} copies of {d}")
+    if which is not None:
+        _dev(which, "which", torch.int32)
+        if which.numel() != n:
+            raise KernelError(f"streams_sum: {which.numel()} rows for {n} outputs")
+    elif rows.shape[0] != n:
+        raise KernelError(f"streams_sum: {rows.shape[0]} tokens for {n} outputs")
+    _check(library().gl3_streams_sum(_ptr(rows), _ptr(which), n, int(S), d, _ptr(out), _stream()), "streams_sum")
+
+
+def latent_prep(proj, col_q, q_rank, col_kv, rank, rot, wq, wkv, eps, positions, table_rows, block_table, cos, sin, cq,
+                k_cache, page_size, H, offsets, pairs):
+    """``proj`` [T, ld] float32 holds the sums of a query latent (``q_rank`` from ``col_q``) and of a key/value latent
+    (``rank`` from ``col_kv``, then ``rot`` elements of a key part that all heads share). ``cq`` [T, q_rank] = the
+    first divided by its root mean square times ``wq``; the token's row of ``k_cache`` [page, 1, page_size, dk] takes
+    [the second the same way with ``wkv`` | the shared part turned in adjacent pairs by the position | zeros].
+    ``offsets`` [H + 1] and ``pairs`` [T H] receive the runs with which ``expert_gemm`` works head by head on rows
+    [T H, *] (row t H + h is head h of token t)."""
+    _f32_rows(proj, "proj", max(col_q + q_rank, col_kv + rank + rot))
+    T = proj.shape[0]
+    _dev(wq, "wq", torch.float32); _dev(wkv, "wkv", torch.float32); _dev(cq, "cq"); _dev(k_cache, "k_cache", cq.dtype)
+    _dev(positions, "positions", torch.int32); _dev(table_rows, "table_rows", torch.int32)
+    _dev(block_table, "block_table", torch.int32); _dev(offsets, "offsets", torch.int32); _dev(pairs, "pairs", torch.int32)
+    if rot:
+        _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rot // 2:
+            raise KernelError(f"latent_prep: table {tuple(cos.shape)} for {rot} rotated elements")
+    if (wq.shape != (q_rank,) or wkv.shape != (rank,) or cq.shape != (T, q_rank) or k_cache.dim() != 4 or k_cache.shape[1] != 1
+            or k_cache.shape[2] != page_size or positions.numel() != T or table_rows.numel() != T or block_table.dim() != 2
+            or offsets.numel() != H + 1 or pairs.numel() != T * H):
+        raise KernelError(f"latent_prep: weights {tuple(wq.shape)}, {tuple(wkv.shape)}; cq {tuple(cq.shape)}; cache "
+                          f"{tuple(k_cache.shape)}; {offsets.numel()} offsets, {pairs.numel()} pairs for {T} tokens of {H} heads")
+    _check(library().gl3_latent_prep(_ptr(proj), proj.stride(0), T, int(col_q), int(q_rank), int(col_kv), int(rank), int(rot),
+                                     _ptr(wq), _ptr(wkv), float(eps), _ptr(positions), _ptr(table_rows), _ptr(block_table),
+                                     block_table.shape[1], _ptr(cos), _ptr(sin), _ptr(cq), _ptr(k_cache), _code(cq, "cq"),
+                                     int(page_size), k_cache.shape[3], int(H), _ptr(offsets), _ptr(pairs), _stream()),
+           "latent_prep")
+
+
+def latent_query(q, H, dim, rot, positions, cos, sin, qa, rank):
+    """``q`` [T, H (dim + rot)]: every head's last ``rot`` elements, turned in adjacent pairs by the token's position,
+    go to columns ``rank .. rank + rot`` of the head's row in ``qa`` [T, H dk], zeros behind them."""
+    _dev(q, "q"); _dev(qa, "qa", q.dtype); _dev(positions, "positions", torch.int32)
+    T = q.shape[0]
+    dk = qa.shape[1] // H
+    if q.shape != (T, H * (dim + rot)) or qa.shape != (T, H * dk) or dk < rank + rot or positions.numel() != T:
+        raise KernelError(f"latent_query: q {tuple(q.shape)}, qa {tuple(qa.shape)} for {H} heads of {dim} + {rot}, latents of {rank}")
+    if rot:
+        _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rot // 2:
+            raise KernelError(f"latent_query: table {tuple(cos.shape)} for {rot} rotated elements")
+    _check(library().gl3_latent_query(_ptr(q), _code(q, "q"), T, int(H), int(dim), int(rot), _ptr(positions), _ptr(cos),
+                                      _ptr(sin), _ptr(qa), int(rank), dk, _stream()), "latent_query")
+
+
+def sigmoid_gate(a, gate, col_g):
+    """``a`` [T, C] *= sigmoid(gate[:, col_g : col_g + C]); the gate's rows are float32."""
+    _dev(a, "a")
+    T, C = a.shape
+    _f32_rows(gate, "gate", col_g + C)
+    if gate.shape[0] != T:
+        raise KernelError(f"sigmoid_gate: {gate.shape[0]} gate rows for {T}")
+    _check(library().gl3_sigmoid_gate(_ptr(a), _code(a, "a"), _ptr(gate), gate.stride(0), int(col_g), T, C, _stream()),
+           "sigmoid_gate")
 
 
 def sides_norm_add(x, a, b, wa, wb, eps, factor, ssq=None, next_weight=None, xg=None):
@@ -1470,11 +1631,12 @@ def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, 
         if part_o.numel() < T * n_heads * n_splits * head_dim or part_ml.numel() < T * n_heads * n_splits * 2:
             raise KernelError("attention: the workspace of the splits is too small")
         floats = T * n_heads * n_splits * (head_dim + 2)
+    has_sink, sink_value, sinks = _sink(sink, n_heads, "attention_decode")
     _check(library().gl3_attention_decode(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
         block_table.shape[1], _ptr(part_o), _ptr(part_ml), floats, _ptr(out), out.stride(0), T, n_heads, n_kv,
         head_dim, page_size, int(window or 0), float(scale), n_splits, _slopes(slopes, n_heads, "attention_decode"),
-        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v,
+        has_sink, sink_value, int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v, sinks,
         _stream()), "attention_decode")
 
 
@@ -1590,11 +1752,12 @@ def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, o
             raise KernelError("attention: one table row per sequence")
     elif block_table.shape[0] < B:
         raise KernelError("attention: the block table has fewer rows than there are sequences")
+    has_sink, sink_value, sinks = _sink(sink, n_heads, "attention_prefill")
     _check(library().gl3_attention_prefill(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(cu_seqlens), _ptr(kv_before), _ptr(block_table),
         _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim,
         page_size, int(window or 0), float(scale), int(wide_from), _slopes(slopes, n_heads, "attention_prefill"),
-        int(sink is not None), float(sink or 0.0), int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v,
+        has_sink, sink_value, int(keep_first or 0) if window else 0, int(chunk or 0), n_kv // n_v, sinks,
         _stream()), "attention_prefill")
 
 

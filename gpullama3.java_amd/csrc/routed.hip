@@ -12,32 +12,48 @@
 // ----------------------------------------------------------------- the choice
 // logits [T][E] float. The `top` largest (the lower number wins a tie) -> idx [T][top]; their weights are the softmax
 // over the chosen logits alone -> wts [T][top]. One thread a token.
+// With `scores` set the rule is another: s = softmax over all E logits; the choice goes by s + correction[e]
+// (correction may be null), the weights are the chosen s themselves divided by their sum plus sum_eps.
 __device__ __forceinline__ void route_choose(const float* __restrict__ logits, int t, int E, int top, int* idx,
-                                             float* __restrict__ wts, int always) {
+                                             float* __restrict__ wts, int always, int scores,
+                                             const float* __restrict__ correction, float sum_eps) {
   const float* z = logits + (long)t * E;
   const int stride = top + (always >= 0 ? 1 : 0);
   int chosen[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
+  float z_max = -INFINITY, z_sum = 1.f;
+  if (scores) {
+    for (int e = 0; e < E; ++e) z_max = fmaxf(z_max, z[e]);
+    z_sum = 0.f;
+    for (int e = 0; e < E; ++e) z_sum += expf(z[e] - z_max);
+  }
   for (int j = 0; j < top; ++j) {
     int best = -1;
-    float bv = -INFINITY;
+    float bv = -INFINITY, bs = 0.f;
     for (int e = 0; e < E; ++e) {
       bool taken = false;
       for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
-      const float v = z[e];
+      const float sc = scores ? expf(z[e] - z_max) / z_sum : z[e];
+      const float v = (scores && correction) ? sc + correction[e] : sc;
       if (!taken && (best < 0 || v > bv)) {
         best = e;
         bv = v;
+        bs = sc;
       }
     }
     chosen[j] = best;
-    val[j] = bv;
+    val[j] = bs;
   }
   float sum = 0.f;
-  const float largest = val[0];          // (the first chosen is the largest)
-  for (int j = 0; j < top; ++j) {
-    val[j] = expf(val[j] - largest);
-    sum += val[j];
+  if (scores) {
+    for (int j = 0; j < top; ++j) sum += val[j];
+    sum += sum_eps;
+  } else {
+    const float largest = val[0];          // (the first chosen is the largest)
+    for (int j = 0; j < top; ++j) {
+      val[j] = expf(val[j] - largest);
+      sum += val[j];
+    }
   }
   for (int j = 0; j < top; ++j) {
     idx[(long)t * stride + j] = chosen[j];
@@ -50,9 +66,10 @@ __device__ __forceinline__ void route_choose(const float* __restrict__ logits, i
 }
 
 __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ logits, int T, int E, int top,
-                                                         int* __restrict__ idx, float* __restrict__ wts, int always) {
+                                                         int* __restrict__ idx, float* __restrict__ wts, int always, int scores,
+                                                         const float* __restrict__ correction, float sum_eps) {
   const int t = blockIdx.x * 64 + threadIdx.x;
-  if (t < T) route_choose(logits, t, E, top, idx, wts, always);
+  if (t < T) route_choose(logits, t, E, top, idx, wts, always, scores, correction, sum_eps);
 }
 
 // ----------------------------------------------------------------- pairs ordered by expert
@@ -89,8 +106,9 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict_
 // Both in one launch for a step of at most 1024 tokens (a thread a token, then the block orders the pairs).
 __global__ __launch_bounds__(1024) void route_few_kernel(const float* __restrict__ logits, int T, int E, int top,
                                                           int* idx, float* __restrict__ wts,
-                                                          int* __restrict__ offsets, int* __restrict__ sorted, int always) {
-  if ((int)threadIdx.x < T) route_choose(logits, threadIdx.x, E, top, idx, wts, always);
+                                                          int* __restrict__ offsets, int* __restrict__ sorted, int always,
+                                                          int scores, const float* __restrict__ correction, float sum_eps) {
+  if ((int)threadIdx.x < T) route_choose(logits, threadIdx.x, E, top, idx, wts, always, scores, correction, sum_eps);
   __threadfence_block();
   __syncthreads();
   const int more = always >= 0 ? 1 : 0;
@@ -100,7 +118,7 @@ __global__ __launch_bounds__(1024) void route_few_kernel(const float* __restrict
 // `always` (-1: none): the number E of one more expert behind the router's, which every token passes with weight 1; idx
 // and wts then have top + 1 entries a token, offsets E + 2.
 extern "C" int gl3_route(const float* logits, int n_tokens, int E, int top, int* idx, float* wts, int* offsets, int* sorted,
-                         int always, hipStream_t stream) {
+                         int always, int scores, const float* correction, float sum_eps, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(logits && idx && wts && offsets && sorted, "gl3_route: null argument");
   const int more = always >= 0 ? 1 : 0;
@@ -108,11 +126,13 @@ extern "C" int gl3_route(const float* logits, int n_tokens, int E, int top, int*
               "gl3_route: the %d largest of %d experts (at most %d of %d)", top, E, ROUTE_MAX_TOP, ROUTE_MAX_EXPERTS);
   GL3_REQUIRE(always < 0 || always == E, "gl3_route: the expert that every token passes is number %d, not %d", E, always);
   if (n_tokens <= 64) {
-    route_few_kernel<<<dim3(1), dim3(1024), 0, stream>>>(logits, n_tokens, E, top, idx, wts, offsets, sorted, always);
+    route_few_kernel<<<dim3(1), dim3(1024), 0, stream>>>(logits, n_tokens, E, top, idx, wts, offsets, sorted, always, scores,
+                                                         correction, sum_eps);
     GL3_LAUNCH_CHECK();
     return 0;
   }
-  route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts, always);
+  route_topk_kernel<<<dim3((n_tokens + 63) / 64), dim3(64), 0, stream>>>(logits, n_tokens, E, top, idx, wts, always, scores,
+                                                                                 correction, sum_eps);
   GL3_LAUNCH_CHECK();
   route_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(idx, n_tokens * (top + more), E + more, offsets, sorted);
   GL3_LAUNCH_CHECK();
@@ -128,6 +148,21 @@ __device__ __forceinline__ float gl3_expert_act(float v, int act) {
   if (act == 2) return gl3_activation<false>(v, GL3_ACT_GELU_TANH);
   if (act == 3) return gl3_activation<false>(v, GL3_ACT_SILU);
   return v;
+}
+
+// A gated expert: the rows of W are gate and up in turns (row 2 n the gate's, row 2 n + 1 the up's row n), so a lane that
+// holds column c of the sums finds its partner's in the lane beside it; the even one writes column c / 2 of the
+// output: act(gate) * (up + shift), both bounded by `limit` first where it is positive (gl3_gated). Every lane of a
+// wave must come here (the partner's value travels from lane to lane); `ok` says whether this lane's element exists.
+template <typename TO>
+__device__ __forceinline__ void expert_store(TO* __restrict__ out, long ldo, int row, int n, bool ok, float v, int act,
+                                             int gate_act, float limit, float shift) {
+  if (gate_act < 0) {
+    if (ok) out[(long)row * ldo + n] = from_f32<TO>(gl3_expert_act(v, act));
+    return;
+  }
+  const float up = __shfl_xor(v, 1, 64);
+  if (ok && !(n & 1)) out[(long)row * ldo + (n >> 1)] = from_f32<TO>(gl3_gated<false>(v, up, gate_act, limit, shift));
 }
 
 __device__ __forceinline__ bool expert_tile(const int* offsets, int E, int n_rows, int TM, int tile, int* e_out, int* lo_out,
@@ -160,7 +195,8 @@ __global__ __launch_bounds__(256) void expert_gemm_generic_kernel(const TA* __re
                                                                    const TW* __restrict__ W, int N, int K,
                                                                    const int* __restrict__ offsets,
                                                                    const int* __restrict__ sorted, int E, int n_rows,
-                                                                   TO* __restrict__ out, long ldo, int act) {
+                                                                   TO* __restrict__ out, long ldo, int act, int gate_act, float limit,
+                                                                   float shift) {
   __shared__ float sa[EG_TM][EG_TK + 1];
   __shared__ float sw[EG_TN][EG_TK + 1];
   __shared__ int rows[EG_TM];
@@ -191,11 +227,10 @@ __global__ __launch_bounds__(256) void expert_gemm_generic_kernel(const TA* __re
     }
     __syncthreads();
   }
-  if (rows[r] < 0) return;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int n = n0 + cg + 16 * j;
-    if (n < N) out[(long)rows[r] * ldo + n] = from_f32<TO>(gl3_expert_act(acc[j], act));
+    expert_store<TO>(out, ldo, rows[r], n, rows[r] >= 0 && n < N, acc[j], act, gate_act, limit, shift);
   }
 }
 
@@ -211,7 +246,8 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __r
                                                                 const bf16_t* __restrict__ W, int N, int K,
                                                                 const int* __restrict__ offsets,
                                                                 const int* __restrict__ sorted, int E, int n_rows,
-                                                                TO* __restrict__ out, long ldo, int act) {
+                                                                TO* __restrict__ out, long ldo, int act, int gate_act, float limit,
+                                                                   float shift) {
   __shared__ int rows[EM_TM];
   int e, lo, hi;
   if (!expert_tile(offsets, E, n_rows, EM_TM, blockIdx.x, &e, &lo, &hi)) return;
@@ -248,13 +284,12 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(const bf16_t* __r
   }
   // a lane holds column li of rows 4 (lane / 16) .. + 3 of every group
   const int nc = blockIdx.y * EM_TN + wave * 16 + li;
-  if (nc >= N) return;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = rows[g * 16 + (lane >> 4) * 4 + i];
-      if (row >= 0) out[(long)row * ldo + nc] = from_f32<TO>(gl3_expert_act(acc[g][i], act));
+      expert_store<TO>(out, ldo, row, nc, row >= 0 && nc < N, acc[g][i], act, gate_act, limit, shift);
     }
   }
 }
@@ -272,7 +307,8 @@ __global__ __launch_bounds__(EF_WAVES * 64) void expert_gemm_few_kernel(const bf
                                                                         const bf16_t* __restrict__ W, int N, int K,
                                                                         const int* __restrict__ offsets,
                                                                         const int* __restrict__ sorted, int E, int n_rows,
-                                                                        TO* __restrict__ out, long ldo, int act) {
+                                                                        TO* __restrict__ out, long ldo, int act, int gate_act, float limit,
+                                                                   float shift) {
   constexpr int TM = 16 * G;
   __shared__ int rows[TM];
   __shared__ float part[EF_WAVES][TM][EF_TN + 1];
@@ -331,13 +367,15 @@ __global__ __launch_bounds__(EF_WAVES * 64) void expert_gemm_few_kernel(const bf
 #pragma unroll
     for (int i = 0; i < 4; ++i) part[wave][g * 16 + (lane >> 4) * 4 + i][li] = acc[g][i];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < m * EF_TN; idx += EF_WAVES * 64) {
-    const int r = idx / EF_TN, c = idx % EF_TN;
+  for (int base = 0; base < m * EF_TN; base += EF_WAVES * 64) {      // (every lane of a wave that has work walks along)
+    const int idx = base + threadIdx.x;
+    const bool in = idx < m * EF_TN;
+    const int r = in ? idx / EF_TN : 0, c = idx % EF_TN;
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < EF_WAVES; ++w) sum += part[w][r][c];
     const int nc = blockIdx.y * EF_TN + c;
-    if (nc < N) out[(long)rows[r] * ldo + nc] = from_f32<TO>(gl3_expert_act(sum, act));
+    expert_store<TO>(out, ldo, rows[r], nc, in && nc < N, sum, act, gate_act, limit, shift);
   }
 }
 
@@ -357,7 +395,8 @@ __global__ __launch_bounds__(512) void expert_gemm_tiled_kernel(const bf16_t* __
                                                                  const bf16_t* __restrict__ W, int N, int K,
                                                                  const int* __restrict__ offsets,
                                                                  const int* __restrict__ sorted, int E, int n_rows,
-                                                                 TO* __restrict__ out, long ldo, int act) {
+                                                                 TO* __restrict__ out, long ldo, int act, int gate_act, float limit,
+                                                                   float shift) {
   constexpr int NT = 512, NA = ET_BM * 8 / NT, NWC = ET_BN * 8 / NT;
   __shared__ __attribute__((aligned(16))) bf16_t As[2][ET_BM][ET_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[2][ET_BN][ET_LD];
@@ -439,21 +478,23 @@ __global__ __launch_bounds__(512) void expert_gemm_tiled_kernel(const bf16_t* __
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     const int row = rows[wm * 32 + (v >> 2) * 8 + lh * 4 + (v & 3)];
-    if (row < 0) continue;
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn) {
       const int n = n0 + wn * 64 + tn * 32 + lr;
-      if (n < N) out[(long)row * ldo + n] = from_f32<TO>(gl3_expert_act(acc[tn][v], act));
+      expert_store<TO>(out, ldo, row, n, row >= 0 && n < N, acc[tn][v], act, gate_act, limit, shift);
     }
   }
 }
 
 extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, const void* W, int w_dtype, int E, int N, int K,
                                const int* offsets, const int* sorted, int n_rows, void* out, int out_dtype, long ldo, int act,
-                               int use_mfma, hipStream_t stream) {
+                               int use_mfma, int gate_act, float limit, float shift, hipStream_t stream) {
   if (n_rows == 0) return 0;
-  GL3_REQUIRE(A && W && out && n_rows > 0 && E >= 1 && N > 0 && K > 0 && a_div >= 1 && lda >= K && ldo >= N,
+  GL3_REQUIRE(A && W && out && n_rows > 0 && E >= 1 && N > 0 && K > 0 && a_div >= 1 && lda >= K &&
+                  ldo >= (gate_act >= 0 ? N / 2 : N),
               "gl3_expert_gemm: bad arguments");
+  GL3_REQUIRE(gate_act < 0 || (GL3_ACT_KNOWN(gate_act) && N % 2 == 0),
+              "gl3_expert_gemm: a gated expert has gate and up rows in turns (%d rows) and a known activation (%d)", N, gate_act);
   GL3_REQUIRE((offsets == nullptr) == (sorted == nullptr) && (offsets || E == 1),
               "gl3_expert_gemm: runs and their pairs come together; without them one expert takes every row");
   GL3_REQUIRE(act >= 0 && act <= 3, "gl3_expert_gemm: unknown activation %d", act);
@@ -466,10 +507,10 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
     const dim3 grid((n_rows + ET_BM - 1) / ET_BM + (offsets ? E : 0), (N + ET_BN - 1) / ET_BN), block(512);
     if (out_dtype == GL3_BF16)
       expert_gemm_tiled_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                   sorted, E, n_rows, (bf16_t*)out, ldo, act);
+                                                                   sorted, E, n_rows, (bf16_t*)out, ldo, act, gate_act, limit, shift);
     else
       expert_gemm_tiled_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                  sorted, E, n_rows, (float*)out, ldo, act);
+                                                                  sorted, E, n_rows, (float*)out, ldo, act, gate_act, limit, shift);
     GL3_LAUNCH_CHECK();
     return 0;
   }
@@ -481,7 +522,7 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
     const dim3 grid((n_rows + 16 * G - 1) / (16 * G) + (offsets ? E : 0), (N + EF_TN - 1) / EF_TN), block(EF_WAVES * 64);
 #define EF_LAUNCH(TO, G)                                                                                                \
   expert_gemm_few_kernel<TO, G><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets, \
-                                                            sorted, E, n_rows, (TO*)out, ldo, act)
+                                                            sorted, E, n_rows, (TO*)out, ldo, act, gate_act, limit, shift)
     if (out_dtype == GL3_BF16) {
       if (G == 1) EF_LAUNCH(bf16_t, 1); else if (G == 2) EF_LAUNCH(bf16_t, 2); else EF_LAUNCH(bf16_t, 4);
     } else {
@@ -496,10 +537,10 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
     const dim3 grid((n_rows + EM_TM - 1) / EM_TM + (offsets ? E : 0), (N + EM_TN - 1) / EM_TN), block(256);
     if (out_dtype == GL3_BF16)
       expert_gemm_mfma_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                  sorted, E, n_rows, (bf16_t*)out, ldo, act);
+                                                                  sorted, E, n_rows, (bf16_t*)out, ldo, act, gate_act, limit, shift);
     else if (out_dtype == GL3_F32)
       expert_gemm_mfma_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)A, lda, a_div, (const bf16_t*)W, N, K, offsets,
-                                                                 sorted, E, n_rows, (float*)out, ldo, act);
+                                                                 sorted, E, n_rows, (float*)out, ldo, act, gate_act, limit, shift);
     else GL3_REQUIRE(false, "gl3_expert_gemm: unknown output dtype %d", out_dtype);
     GL3_LAUNCH_CHECK();
     return 0;
@@ -507,7 +548,7 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
   const dim3 grid((n_rows + EG_TM - 1) / EG_TM + (offsets ? E : 0), (N + EG_TN - 1) / EG_TN), block(256);
 #define EG_LAUNCH(TA, TW, TO)                                                                                          \
   expert_gemm_generic_kernel<TA, TW, TO><<<grid, block, 0, stream>>>((const TA*)A, lda, a_div, (const TW*)W, N, K, offsets, \
-                                                                     sorted, E, n_rows, (TO*)out, ldo, act)
+                                                                     sorted, E, n_rows, (TO*)out, ldo, act, gate_act, limit, shift)
   if (a_dtype == GL3_F32 && w_dtype == GL3_F32 && out_dtype == GL3_F32) EG_LAUNCH(float, float, float);
   else if (a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && out_dtype == GL3_BF16) EG_LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (a_dtype == GL3_BF16 && w_dtype == GL3_BF16 && out_dtype == GL3_F32) EG_LAUNCH(bf16_t, bf16_t, float);
@@ -518,25 +559,38 @@ extern "C" int gl3_expert_gemm(const void* A, int a_dtype, long lda, int a_div, 
 }
 
 // ----------------------------------------------------------------- the weighted sum
-// out[t] (+)= sum_j wts[t][j] * y[t * top + j], j in order. One thread an element.
+// out[t] (+)= sum_j wts[t][j] * y[t * top + j], j in order. One thread an element. With idx [T][top] and n_real: a pair
+// whose expert number is n_real or more is an identity expert, whose output is the token's input row h[t] itself (y
+// holds nothing for it).
+template <typename TH>
 __global__ void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ wts, int top, int d,
-                                     float* __restrict__ out, int accumulate, long n) {
+                                     float* __restrict__ out, int accumulate, long n, const int* __restrict__ idx,
+                                     int n_real, const TH* __restrict__ h) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const long t = i / d;
   const int c = i % d;
   float s = accumulate ? out[i] : 0.f;
-  for (int j = 0; j < top; ++j) s = fmaf(wts[t * top + j], y[(t * top + j) * d + c], s);
+  for (int j = 0; j < top; ++j) {
+    const float v = (idx && idx[t * top + j] >= n_real) ? to_f32<TH>(h[t * d + c]) : y[(t * top + j) * d + c];
+    s = fmaf(wts[t * top + j], v, s);
+  }
   out[i] = s;
 }
 
 extern "C" int gl3_route_combine(const float* y, const float* wts, int n_tokens, int top, int d, float* out, int accumulate,
-                                 hipStream_t stream) {
+                                 const int* idx, int n_real, const void* h, int h_dtype, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(y && wts && out && n_tokens > 0 && top >= 1 && d > 0, "gl3_route_combine: bad arguments");
+  GL3_REQUIRE((idx == nullptr) == (h == nullptr), "gl3_route_combine: identity experts need the choices and the input rows");
   const long n = (long)n_tokens * d;
   GL3_REQUIRE((n + 255) / 256 < (1L << 31), "gl3_route_combine: too many elements");
-  route_combine_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(y, wts, top, d, out, accumulate, n);
+  if (h && h_dtype == GL3_BF16)
+    route_combine_kernel<bf16_t><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(y, wts, top, d, out, accumulate, n,
+                                                                                            idx, n_real, (const bf16_t*)h);
+  else
+    route_combine_kernel<float><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(y, wts, top, d, out, accumulate, n,
+                                                                                           idx, n_real, (const float*)h);
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -127,7 +127,11 @@ struct ScanArgs {
   float* piece_state;                         // [sequence][piece][H][N][P]
   float* piece_decay;                         // [sequence][piece][H]
   int n_pieces, piece_len;
+  int act;                                    // 1: q, k and v pass silu as they are read (a linear attention whose
+                                              // projections carry an activation); 0: as they are
 };
+
+__device__ __forceinline__ float scan_in(float v, int act) { return act ? v / (1.0f + expf(-v)) : v; }
 
 template <int NR, int MODE>
 __global__ void decay_scan_kernel(ScanArgs A) {
@@ -164,12 +168,12 @@ __global__ void decay_scan_kernel(ScanArgs A) {
     for (int e = threadIdx.x; e < m * NP; e += blockDim.x) {
       const int j = e / NP, i = e % NP;
       const long t = first + base + j;
-      sk[e] = i < N ? A.k[t * A.ld_k + A.col_k + g * N + i] : 0.f;
-      if (MODE != 1) sq[e] = i < N ? A.q[t * A.ld_q + A.col_q + g * N + i] : 0.f;
+      sk[e] = i < N ? scan_in(A.k[t * A.ld_k + A.col_k + g * N + i], A.act) : 0.f;
+      if (MODE != 1) sq[e] = i < N ? scan_in(A.q[t * A.ld_q + A.col_q + g * N + i], A.act) : 0.f;
     }
     for (int e = threadIdx.x; e < m * pt; e += blockDim.x) {
       const int j = e / pt, i = e % pt, col = blockIdx.z * pt + i;
-      sv[j * pt + i] = col < P ? A.v[(long)(first + base + j) * A.ld_v + A.col_v + h * P + col] : 0.f;
+      sv[j * pt + i] = col < P ? scan_in(A.v[(long)(first + base + j) * A.ld_v + A.col_v + h * P + col], A.act) : 0.f;
     }
     for (int j = threadIdx.x; j < m; j += blockDim.x) {
       const long t = first + base + j;
@@ -243,7 +247,7 @@ extern "C" int gl3_decay_scan(const float* q, long ld_q, int col_q, const float*
                               long ld_v, int col_v, const float* a_tok, const float* b_tok, long ld_ab, const float* a_head,
                               float b_const, float* state, long state_ld, long state_off, const int* cu_seqlens,
                               const int* slot_ids, float* out, long ld_o, int n_seqs, int H, int heads_per_group, int N, int P,
-                              float* pieces, long pieces_floats, int max_len, int piece_len, hipStream_t stream) {
+                              float* pieces, long pieces_floats, int max_len, int piece_len, int act, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   GL3_REQUIRE(q && k && v && state && cu_seqlens && slot_ids && out && (a_tok || a_head), "gl3_decay_scan: null argument");
   GL3_REQUIRE(n_seqs > 0 && H > 0 && H <= 65535 && heads_per_group > 0 && H % heads_per_group == 0 && N > 0 && N <= 1024 && P > 0,
@@ -273,7 +277,7 @@ extern "C" int gl3_decay_scan(const float* q, long ld_q, int col_q, const float*
   while (round > 1 && (bytes(round) > 60000 || (round * pt) % 4)) round /= 2;
   GL3_REQUIRE(bytes(round) <= 64000, "gl3_decay_scan: keys of %d with values of %d do not fit shared memory", N, P);
   ScanArgs A{q, ld_q, col_q, k, ld_k, col_k, v, ld_v, col_v, a_tok, b_tok, ld_ab, a_head, b_const, state, state_ld, state_off,
-             cu_seqlens, slot_ids, out, ld_o, H, heads_per_group, N, P, R, round, nullptr, nullptr, 1, 0};
+             cu_seqlens, slot_ids, out, ld_o, H, heads_per_group, N, P, R, round, nullptr, nullptr, 1, 0, act ? 1 : 0};
   const int ptiles = (P + pt - 1) / pt;
   const dim3 block(R * pt);
   const size_t sh = bytes(round);
@@ -316,7 +320,8 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __res
                                                                long ld_x, int col_x, const float* __restrict__ skip_d,
                                                                int head_dim, const float* __restrict__ gate, long ld_g,
                                                                int col_g, const float* __restrict__ w, float eps,
-                                                               int gate_first, int C, int gsize, TO* __restrict__ out) {
+                                                               int gate_first, int C, int gsize, TO* __restrict__ out,
+                                                               int gate_sigmoid) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const int c0 = blockIdx.y * gsize;
@@ -327,7 +332,7 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __res
     if (skip_d) y = fmaf(skip_d[c / head_dim], skip_x[t * ld_x + col_x + c], y);
     if (gate_first) {
       const float g = gate[t * ld_g + col_g + c];
-      y *= g / (1.0f + expf(-g));
+      y *= (gate_sigmoid ? 1.0f : g) / (1.0f + expf(-g));
     }
     ss += y * y;
   }
@@ -338,7 +343,7 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __res
     float y = o[t * C + c];
     if (skip_d) y = fmaf(skip_d[c / head_dim], skip_x[t * ld_x + col_x + c], y);
     const float g = gate[t * ld_g + col_g + c];
-    const float sg = g / (1.0f + expf(-g));
+    const float sg = (gate_sigmoid ? 1.0f : g) / (1.0f + expf(-g));      // silu of the gate, or its sigmoid
     y = gate_first ? y * sg * inv : y * inv * sg;
     if (w) y *= w[c];
     out[t * C + c] = from_f32<TO>(y);
@@ -347,7 +352,8 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __res
 
 extern "C" int gl3_group_norm_gate(const float* o, const float* skip_x, long ld_x, int col_x, const float* skip_d, int head_dim,
                                    const float* gate, long ld_g, int col_g, const float* w, float eps, int gate_first,
-                                   int n_tokens, int C, int gsize, void* out, int out_dtype, hipStream_t stream) {
+                                   int n_tokens, int C, int gsize, void* out, int out_dtype, int gate_sigmoid,
+                                   hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(o && gate && out && n_tokens > 0 && C > 0 && gsize > 0 && C % gsize == 0 && C / gsize <= 65535,
               "gl3_group_norm_gate: %d channels in groups of %d", C, gsize);
@@ -358,10 +364,10 @@ extern "C" int gl3_group_norm_gate(const float* o, const float* skip_x, long ld_
   const dim3 grid(n_tokens, C / gsize), block(threads);
   if (out_dtype == GL3_F32)
     group_norm_gate_kernel<float><<<grid, block, 0, stream>>>(o, skip_x, ld_x, col_x, skip_d, head_dim, gate, ld_g, col_g, w, eps,
-                                                              gate_first, C, gsize, (float*)out);
+                                                              gate_first, C, gsize, (float*)out, gate_sigmoid);
   else if (out_dtype == GL3_BF16)
     group_norm_gate_kernel<bf16_t><<<grid, block, 0, stream>>>(o, skip_x, ld_x, col_x, skip_d, head_dim, gate, ld_g, col_g, w, eps,
-                                                               gate_first, C, gsize, (bf16_t*)out);
+                                                               gate_first, C, gsize, (bf16_t*)out, gate_sigmoid);
   else GL3_REQUIRE(false, "gl3_group_norm_gate: unknown dtype %d", out_dtype);
   GL3_LAUNCH_CHECK();
   return 0;

@@ -1,0 +1,136 @@
+// Several copies of the residual row per token ("streams"), mixed by learned numbers around every sublayer.
+//
+// rows [T][S][d] float: token t's S copies one after another. Around a sublayer with the numbers in[S], mix[S][S]
+// (indexed [from][to]) and out[S]:
+//   the sublayer reads  u = sum_s in[s] x_s          (through an RMS norm: h = u / sqrt(mean(u^2) + eps) * w)
+//   and leaves          x_r <- sum_s mix[s][r] x_s + out[r] * y     for all r at once from the old copies.
+// One kernel does both ends that meet between two sublayers: it takes the output y of the sublayer before (if any),
+// writes the new copies, and makes the input h of the sublayer behind (if any) from them, so the copies make one
+// trip to memory per sublayer. Everything is 32-bit arithmetic; h takes the activations' type. The sums run in the
+// order of s, and a row's sum of squares in an order that the width alone fixes.
+#include "common.h"
+
+#define STREAMS_MAX 8
+
+template <typename TO>
+__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ rows, int S, int d,
+                                                            const float* __restrict__ y, const float* __restrict__ mix,
+                                                            const float* __restrict__ out_w,
+                                                            const float* __restrict__ in_w,
+                                                            const float* __restrict__ norm_w, float eps,
+                                                            TO* __restrict__ h) {
+  extern __shared__ float u_row[];           // [d] the mixture that the next sublayer reads
+  __shared__ float scratch[16];
+  __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
+  const long t = blockIdx.x;
+  if (threadIdx.x < S * S && y) s_mix[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    if (y) s_out[threadIdx.x] = out_w[threadIdx.x];
+    if (in_w) s_in[threadIdx.x] = in_w[threadIdx.x];
+  }
+  __syncthreads();
+  float* xr = rows + t * S * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float x[STREAMS_MAX];
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s) x[s] = s < S ? xr[(long)s * d + c] : 0.f;
+    if (y) {
+      const float yv = y[t * d + c];
+      float nx[STREAMS_MAX];
+#pragma unroll
+      for (int r = 0; r < STREAMS_MAX; ++r) {
+        if (r < S) {
+          float v = 0.f;
+#pragma unroll
+          for (int s = 0; s < STREAMS_MAX; ++s)
+            if (s < S) v = fmaf(s_mix[s * S + r], x[s], v);
+          nx[r] = fmaf(s_out[r], yv, v);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < STREAMS_MAX; ++r)
+        if (r < S) {
+          x[r] = nx[r];
+          xr[(long)r * d + c] = nx[r];
+        }
+    }
+    if (in_w) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < STREAMS_MAX; ++s)
+        if (s < S) u = fmaf(s_in[s], x[s], u);
+      u_row[c] = u;
+      ss = fmaf(u, u, ss);
+    }
+  }
+  if (!in_w) return;
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += blockDim.x) h[t * d + c] = from_f32<TO>(u_row[c] * inv * norm_w[c]);
+}
+
+// y null: nothing is added and the copies stay (the first sublayer of a step). in_w null: nothing is read (behind the
+// last sublayer). norm_w: float [d].
+extern "C" int gl3_streams_step(float* rows, int n_tokens, int S, int d, const float* y, const float* mix, const float* out_w,
+                                const float* in_w, const float* norm_w, float eps, void* h, int h_dtype, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(rows && n_tokens > 0 && S >= 1 && S <= STREAMS_MAX && d > 0, "gl3_streams_step: %d tokens with %d copies (at most %d) of %d",
+              n_tokens, S, STREAMS_MAX, d);
+  GL3_REQUIRE(!y || (mix && out_w), "gl3_streams_step: a sublayer's output comes with the numbers that mix it in");
+  GL3_REQUIRE(!in_w || (norm_w && h), "gl3_streams_step: the next sublayer's input needs its norm's weight and a place");
+  GL3_REQUIRE(y || in_w, "gl3_streams_step: nothing to do");
+  const size_t sh = in_w ? (size_t)d * sizeof(float) : 0;
+  GL3_REQUIRE(sh <= 64000, "gl3_streams_step: rows of %d do not fit shared memory", d);
+  const dim3 grid(n_tokens), block(256);
+  if (!in_w || h_dtype == GL3_F32)
+    streams_step_kernel<float><<<grid, block, sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (float*)h);
+  else if (h_dtype == GL3_BF16)
+    streams_step_kernel<bf16_t><<<grid, block, sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (bf16_t*)h);
+  else GL3_REQUIRE(false, "gl3_streams_step: unknown dtype %d", h_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// Every copy of a token's row takes the values of src [T][d] (a step's beginning: the embedding's output).
+__global__ void streams_fill_kernel(const float* __restrict__ src, float* __restrict__ rows, int S, int d, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long t = i / d;
+  const int c = i % d;
+  const float v = src[i];
+  for (int s = 0; s < S; ++s) rows[(t * S + s) * d + c] = v;
+}
+
+extern "C" int gl3_streams_fill(const float* src, float* rows, int n_tokens, int S, int d, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(src && rows && n_tokens > 0 && S >= 1 && d > 0, "gl3_streams_fill: bad arguments");
+  const long n = (long)n_tokens * d;
+  GL3_REQUIRE((n + 255) / 256 < (1L << 31), "gl3_streams_fill: too many elements");
+  streams_fill_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(src, rows, S, d, n);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[r] = the sum of the copies of token which[r] (which null: token r), in the order of the copies.
+__global__ void streams_sum_kernel(const float* __restrict__ rows, const int* __restrict__ which, int S, int d,
+                                   float* __restrict__ out, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long r = i / d;
+  const int c = i % d;
+  const long t = which ? which[r] : r;
+  float v = 0.f;
+  for (int s = 0; s < S; ++s) v += rows[(t * S + s) * d + c];
+  out[i] = v;
+}
+
+extern "C" int gl3_streams_sum(const float* rows, const int* which, int n_out, int S, int d, float* out, hipStream_t stream) {
+  if (n_out == 0) return 0;
+  GL3_REQUIRE(rows && out && n_out > 0 && S >= 1 && d > 0, "gl3_streams_sum: bad arguments");
+  const long n = (long)n_out * d;
+  GL3_REQUIRE((n + 255) / 256 < (1L << 31), "gl3_streams_sum: too many elements");
+  streams_sum_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(rows, which, S, d, out, n);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

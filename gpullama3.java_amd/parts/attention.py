@@ -19,7 +19,10 @@ attention, one kernel that turns the output back and applies the gate. On the sa
 head in front of the rotation (``qk_norm_eps``, in the kernel that turns them), a chunked mask (``chunk``), differential
 attention (``differential``: two score maps per head over the same values; queries and keys then have twice the heads,
 stored head by head as [map 1, map 2], and the cache keeps twice the key heads beside the value heads), and a mixer
-without keys and values of its own (no ``k`` among its names) that only ever reads another entry's.
+without keys and values of its own (no ``k`` among its names) that only ever reads another entry's; a learned sink per
+query head (a stored [n_heads] vector named ``sink``, on every kernel that knows a sink); and values that are the keys
+as projected (``values_are_keys``: no value projection; the key rows stand twice in the stacked product, once to be
+normed and turned, once to be cached as they are).
 """
 from __future__ import annotations
 
@@ -56,13 +59,17 @@ class GQAAttention:
         self.qk_norm_eps = getattr(spec, "qk_norm_eps", None)
         self.chunk = int(getattr(spec, "chunk", None) or 0) or None
         self.reads_only = "k" not in spec.names
+        self.values_are_keys = bool(getattr(spec, "values_are_keys", False))
+        if self.values_are_keys and (self.reads_only or self.vd != self.hs or "v" in spec.names):
+            raise ValueError("an attention whose values are its keys has keys of its own, values of their size and no "
+                             "value projection")
         if self.chunk and spec.window:
             raise ValueError("an attention has a window or a chunked mask, not both")
         # (rotated values, a gate per head, a rotation with values of another size, a norm on queries and keys, several
         # score maps and a mixer that only reads run on the kernels for any sizes)
         self.general = bool(self.value_position_spec is not None or self.gated
                             or (spec.position is not None and self.vd != self.hs) or self.qk_norm_eps is not None
-                            or self.diff is not None or self.reads_only)
+                            or self.diff is not None or self.reads_only or self.values_are_keys)
         if spec.position is None or self.general:
             # (a rotation touches a head's first elements only: zeros behind them stay zeros)
             self.hs, self.vd = -(-self.hs // 16) * 16, -(-self.vd // 16) * 16
@@ -70,6 +77,7 @@ class GQAAttention:
         self.keep_first = int(getattr(spec, "keep_first", 0) or 0) if spec.window else 0
         self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.sink = getattr(spec, "sink", None)
+        self.sink_name = spec.names.get("sink")       # a stored sink per head takes the place of the constant
         bias = getattr(spec, "distance_bias", None)
         self._slopes_host = bias.slopes(self.H) if bias is not None else None
         self.slopes = None
@@ -92,7 +100,11 @@ class GQAAttention:
         n, d, hs, vd = self.names, self.d, self.hs_stored, self.vd_stored
         out = {n["q"]: TensorSpec((self.Hq * hs, d)), n["o"]: TensorSpec((d, self.H * vd))}
         if not self.reads_only:
-            out.update({n["k"]: TensorSpec((self.Kq * hs, d)), n["v"]: TensorSpec((self.Kh * vd, d))})
+            out[n["k"]] = TensorSpec((self.Kq * hs, d))
+            if not self.values_are_keys:
+                out[n["v"]] = TensorSpec((self.Kh * vd, d))
+        if self.sink_name:
+            out[self.sink_name] = TensorSpec((self.H,), "vector", 0.0, 1.0)
         if self.qk_norm_eps is not None:
             out[n["q_norm"]] = TensorSpec((hs,), "vector")
             if not self.reads_only:
@@ -153,6 +165,8 @@ class GQAAttention:
             self.slopes = torch.tensor(self._slopes_host, dtype=torch.float64).to(torch.float32).to(self.w_qkv.device)
 
     def _load_scales(self, weights):
+        if self.sink_name:
+            self.sink = weights[self.sink_name].float().contiguous()
         if self.out_scale_name:
             self.out_scale = weights[self.out_scale_name].float().contiguous()
         if self.out_mult != 1.0:      # the constant rides in the output projection's epilogue with the factor per channel
@@ -167,15 +181,18 @@ class GQAAttention:
             raise ValueError("an attention with rotated values or a gate per head is built without biases")
         if self.reads_only and self.gated:
             raise ValueError("an attention without keys and values of its own is built without a gate per head")
-        kinds = ("q",) if self.reads_only else ("q", "k", "v")
+        kinds = ("q",) if self.reads_only else ("q", "k", "k") if self.values_are_keys else ("q", "k", "v")
         parts = [weights[n[k]] for k in kinds] + ([weights[n["head_gate"]]] if self.gated else [])
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         rows = sum(p.shape[0] for p in parts)
         pad = torch.zeros((-(-rows // 16) * 16 - rows, self.d), dtype=dt, device=parts[0].device)
         self.w_qkv = torch.cat([p.to(dt) for p in parts] + [pad], dim=0).contiguous()
         lo = 0
+        named = set()
         for k, p in zip(kinds + ("head_gate",), parts):      # the stored names stay addressable as views
-            weights[n[k]] = self.w_qkv[lo:lo + p.shape[0]]
+            if k not in named:                                # (key rows that stand twice: the first ones)
+                weights[n[k]] = self.w_qkv[lo:lo + p.shape[0]]
+                named.add(k)
             lo += p.shape[0]
         without = getattr(self, "without", frozenset())
         ops.for_few_rows(self.w_qkv, without=without)

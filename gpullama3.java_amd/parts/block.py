@@ -5,7 +5,10 @@ stream keeps the sum (J/inference/InferenceCore.java:74, :151, :154, :172).
 """
 from __future__ import annotations
 
+import torch
+
 from ..csrc import lib as K
+from ..weights.loader import TensorSpec
 from . import ops
 from .base import build_part, register_part
 
@@ -141,6 +144,83 @@ class OutNormBlock:
             self.ffn_norm.add_into(ctx, x, y, cast)
 
 
+class _StreamNumbers:
+    """The numbers that mix the copies of the residual row around one block's sublayers: per sublayer ``in`` [S],
+    ``mix`` [S, S] (from, to) and ``out`` [S], kept in 32-bit."""
+    graph_safe = True
+
+    def __init__(self, S, names):
+        self.S, self.names = S, names
+        self.values = {}
+
+    def tensors(self):
+        shapes = {"in": (self.S,), "mix": (self.S, self.S), "out": (self.S,)}
+        # (random weights: around 1 / S for what is read, around the identity for what is kept)
+        out = {}
+        for key, name in self.names.items():
+            kind = key.split("_")[1]
+            out[name] = TensorSpec(shapes[kind], "vector", {"in": 1.0 / self.S, "mix": 1.0 / self.S, "out": 1.0}[kind], 0.2)
+        return out
+
+    def load(self, weights):
+        self.values = {key: weights[name].float().contiguous() for key, name in self.names.items()}
+
+    def of(self, sublayer):
+        return tuple(self.values[f"{sublayer}_{k}"] for k in ("in", "mix", "out"))
+
+
+class StreamsBlock:
+    """Every token has S copies of its residual row, ``x`` [T, S d]. A sublayer reads ``norm(sum_s in[s] x_s)`` and
+    its output y goes back as ``x_r <- sum_s mix[s, r] x_s + out[r] y``. One kernel (``lib.streams_step``) does the
+    write-back of one sublayer and the read of the next; the block's first read is its own launch (the block before
+    ends with its write-back: a block may be run more than once, or in another order, so nothing is carried across
+    blocks). Mixer and feed-forward write their output to a 32-bit buffer (``epilogue=EPI_STORE``). The block has no
+    ``first_norm``: the decoder hands it whole rows and folds no norm into a product while it runs."""
+
+    def __init__(self, spec, dtype, device):
+        self.dtype, self.S = dtype, int(spec.streams)
+        self.mixer_norm = build_part("norm", spec.mixer_norm, dtype=dtype)
+        self.mixer = build_part("mixer", spec.mixer, dtype=dtype, device=device)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, dtype=dtype) if spec.ffn is not None else None
+        self.ffn = build_part("ffn", spec.ffn, dtype=dtype, device=device) if spec.ffn is not None else None
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and not getattr(n, "folds", False):
+                raise ValueError(f"the norm in front of a sublayer that reads several copies is weight * x / rms; "
+                                 f"{type(n).__name__} is not")
+        self.numbers = _StreamNumbers(self.S, spec.stream_names)
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.numbers) if p is not None]
+
+    def cache_needs(self):
+        return self.mixer.kv_need(), self.mixer.state_need()
+
+    def forward(self, ctx, x, run):
+        T, d = x.shape[0], x.shape[1] // self.S
+        h = ctx.buffer("streams_input", (T, d), self.dtype)
+        y = ctx.buffer("sublayer_out", (T, d), torch.float32)
+        watch = getattr(ctx.engine, "after_sublayer", None)      # a caller that looks at a sublayer's output and at the rows behind it
+        m_in, m_mix, m_out = self.numbers.of("mixer")
+        K.streams_step(x, self.S, in_w=m_in, norm_w=self.mixer_norm.weight_f32, eps=self.mixer_norm.eps, h=h)
+        self.mixer.forward(ctx, h, y, run, epilogue=ops.EPI_STORE)
+        if watch is not None:
+            watch(run.entry, "mixer", y)
+        if self.ffn is None:
+            K.streams_step(x, self.S, y=y, mix=m_mix, out_w=m_out)
+        else:
+            f_in, f_mix, f_out = self.numbers.of("ffn")
+            K.streams_step(x, self.S, y=y, mix=m_mix, out_w=m_out, in_w=f_in, norm_w=self.ffn_norm.weight_f32,
+                           eps=self.ffn_norm.eps, h=h)
+            if watch is not None:
+                watch(run.entry, "mixer_added", x)
+            self.ffn.forward(ctx, h, y, epilogue=ops.EPI_STORE)
+            if watch is not None:
+                watch(run.entry, "ffn", y)
+            K.streams_step(x, self.S, y=y, mix=f_mix, out_w=f_out)
+        ops.residual_written(ctx, x)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "streams", StreamsBlock)
 register_part("block", "outnorm", OutNormBlock)
 register_part("block", "parallel", ParallelBlock)

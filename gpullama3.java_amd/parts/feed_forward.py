@@ -80,9 +80,11 @@ class GatedFeedForward:
         out = type("Out", (), {"dtype": self.dtype, "shape": (h.shape[0], self.F)})
         return self.b_gate_up is None and ops.takes_folded_norm(h, self.w_gate_up, out, ops.EPI_GATED)
 
-    def forward(self, ctx, h, x):
+    def forward(self, ctx, h, x, epilogue=ops.EPI_ADD):
+        """``epilogue``: EPI_ADD adds the output into the residual rows ``x``; EPI_STORE writes it to ``x``, a float32
+        buffer of the caller's."""
         plain = not self.limit and not self.up_shift and self.out_scale is None and self.act in K.FAST_ACTIVATIONS
-        if (plain and self.b_gate_up is None and self.b_down is None
+        if (plain and self.b_gate_up is None and self.b_down is None and epilogue == ops.EPI_ADD
                 and ops.packs_rows(ctx, h, self.w_gate_up, self.w_down, x)):
             act = ctx.buffer("ffn_act_packed", (-(-self.F // 64), 64, 8), self.dtype)
             ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, act=self.act, pack_out=True)
@@ -91,7 +93,7 @@ class GatedFeedForward:
         act = ctx.buffer("ffn_act", (h.shape[0], self.F), self.dtype)
         ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, bias=self.b_gate_up, act=self.act, act_limit=self.limit,
                    act_shift=self.up_shift)
-        ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, bias=self.b_down, col_scale=self.out_scale)
+        ops.linear(act, self.w_down, x, epilogue, ctx, bias=self.b_down, col_scale=self.out_scale)
 
 
 register_part("ffn", "gated", GatedFeedForward)

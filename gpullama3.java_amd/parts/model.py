@@ -171,6 +171,7 @@ class DecoderModel:
 
     def forward(self, ctx, want_rows):
         """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
+        S = int(getattr(self.spec, "streams", 1) or 1)      # copies of the residual row per token
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
         ctx.ssq = ctx.pending = ctx.next_norm = None   # a context may run more than one forward pass: nothing is left over
         ctx.token_facts, ctx.token_tables = {}, {}
@@ -201,6 +202,11 @@ class DecoderModel:
             ops.residual_written(ctx, x, ssq, 1, xg, firsts[0])
         else:
             K.embed(self.embedding, ctx.token_ids, x, **around)
+            ops.residual_written(ctx, x)
+        if S > 1:
+            # every copy starts as the embedding's output; the blocks work on all of them, [T, S d]
+            one, x = x, ctx.buffer("residual_copies", (ctx.n_tokens, S * self.spec.hidden), torch.float32)
+            K.streams_fill(one, x, S)
             ops.residual_written(ctx, x)
         embedded = None
         if getattr(self, "keeps_embedding", False):
@@ -244,13 +250,23 @@ class DecoderModel:
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:
+            if S > 1:
+                # the copies' sum at the wanted rows is what the final norm and the head read
+                ops.settle_residual(ctx, x)
+                copies, x = x, ctx.buffer("residual_wanted", (n, self.spec.hidden), torch.float32)
+                K.streams_sum(copies, S, x, which=want_rows)
+                want_rows = None                       # (every row of x, in order)
+                ops.residual_written(ctx, x)
             if self.final_norm is not None:
                 h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
             else:
                 # a decoder without a final norm: the head reads the wanted rows as they are
                 ops.settle_residual(ctx, x)
                 h = ctx.buffer("head_rows", (n, self.spec.hidden), self.dtype)
-                K.gather_rows(x, want_rows, h)
+                if want_rows is None:
+                    K.cast_rows(x, h)
+                else:
+                    K.gather_rows(x, want_rows, h)
             ops.linear(h, self.head, logits, ops.EPI_STORE, ctx, bias=self.head_bias)
             if self.spec.logit_scale is not None:
                 K.scale_(logits, self.spec.logit_scale)

@@ -13,6 +13,11 @@ One product makes q, k, v and the gate (rows stacked, padded with zero rows to a
 (``csrc/scan.hip``), which the state space shares: it walks a step's tokens in order from the slot's state (a long
 step as pieces side by side, joined through their start states), so every cut of a sequence into steps gives the same
 result up to 32-bit rounding.
+
+What other linear attentions of this form change, all from the description: the factor on k (``key_scale``), silu on q,
+k and v behind their projections (``input_activation``, applied in 32-bit as the recurrence reads them), no rotation
+(``position`` None), the unit norm over all heads' read-outs together with a stored weight (``norm_over = "all"``), and
+the sigmoid of the gate projection in place of its silu (``gate_activation``).
 """
 from __future__ import annotations
 
@@ -42,12 +47,24 @@ class Retention:
         self.position = build_part("position", spec.position, device=device) if spec.position is not None else None
         self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.device = device
-        self.w_in = self.w_o = self.decay = self.out_scale = None
+        key_scale = getattr(spec, "key_scale", None)
+        self.key_scale = float(self.D) ** -0.5 if key_scale is None else float(key_scale)
+        self.input_activation = getattr(spec, "input_activation", None)
+        self.norm_over = getattr(spec, "norm_over", "head")
+        self.gate_activation = getattr(spec, "gate_activation", "silu")
+        if self.input_activation not in (None, "silu") or self.norm_over not in ("head", "all") \
+                or self.gate_activation not in ("silu", "sigmoid"):
+            raise ValueError(f"a retention with input activation {self.input_activation!r}, a norm over {self.norm_over!r} "
+                             f"and a gate's {self.gate_activation!r} is not built")
+        self.w_in = self.w_o = self.decay = self.out_scale = self.norm_weight = None
 
     def tensors(self):
         n, d, HD, HV = self.names, self.d, self.H * self.D, self.H * self.Dv
-        return {n["q"]: TensorSpec((HD, d)), n["k"]: TensorSpec((HD, d)), n["v"]: TensorSpec((HV, d)),
-                n["g"]: TensorSpec((HV, d)), n["o"]: TensorSpec((d, HV))}
+        out = {n["q"]: TensorSpec((HD, d)), n["k"]: TensorSpec((HD, d)), n["v"]: TensorSpec((HV, d)),
+               n["g"]: TensorSpec((HV, d)), n["o"]: TensorSpec((d, HV))}
+        if self.norm_over == "all":
+            out[n["norm"]] = TensorSpec((HV,), "vector")
+        return out
 
     def load(self, weights):
         n = self.names
@@ -66,6 +83,8 @@ class Retention:
         self.decay = torch.tensor(self.spec.decay, dtype=torch.float64).to(torch.float32).to(dev)
         if self.out_mult != 1.0:      # the constant rides in the output projection's epilogue as a factor per column
             self.out_scale = torch.full((self.d,), self.out_mult, dtype=torch.float32, device=dev)
+        if self.norm_over == "all":
+            self.norm_weight = weights[n["norm"]].float().contiguous()
 
     def kv_need(self):
         return None
@@ -85,9 +104,11 @@ class Retention:
             K.rotate_heads(proj, ctx.positions, [(self.off_q, H, D) + rot, (self.off_k, H, D) + rot], adjacent=pos.adjacent)
         o = ctx.buffer("retention_readout", (T, H * Dv), torch.float32)
         K.decay_scan(proj, self.off_q, proj, self.off_k, proj, self.off_v, ctx.slot_state(run.entry), 0, ctx.cu_seqlens,
-                     ctx.slot_ids, o, H, 1, D, Dv, a_head=self.decay, b_const=float(D) ** -0.5, **ops.scan_pieces(ctx, H, D, Dv))
+                     ctx.slot_ids, o, H, 1, D, Dv, a_head=self.decay, b_const=self.key_scale,
+                     silu_inputs=self.input_activation == "silu", **ops.scan_pieces(ctx, H, D, Dv))
         y = ctx.buffer("retention_out", (T, H * Dv), self.dtype)
-        K.group_norm_gate(o, proj, self.off_g, y, Dv, self.spec.norm_eps)
+        K.group_norm_gate(o, proj, self.off_g, y, Dv if self.norm_over == "head" else H * Dv, self.spec.norm_eps,
+                          weight=self.norm_weight, gate_act=self.gate_activation)
         ops.linear(y, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)
 
 

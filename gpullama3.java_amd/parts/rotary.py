@@ -19,11 +19,29 @@ from .base import register_part
 _F = np.float32
 
 
+def magnitude(scaling):
+    """The factor on cos and sin: ``0.1 ln(factor) + 1`` for the ramp over pair numbers, 1 otherwise."""
+    return 0.1 * math.log(scaling.factor) + 1.0 if hasattr(scaling, "fast") else 1.0
+
+
+def _ramp_ends(head_dim, theta, scaling):
+    """The pair numbers between which a ``YarnRopeScaling`` goes from the plain frequency to the divided one."""
+    def pair_of(turns):
+        return head_dim * math.log(scaling.original_max_position / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+    lo = max(math.floor(pair_of(scaling.fast)), 0)
+    hi = min(math.ceil(pair_of(scaling.slow)), head_dim - 1)
+    return lo, hi
+
+
 def frequencies(head_dim, theta, scaling):
     out = np.zeros(head_dim // 2, dtype=_F)
+    ends = _ramp_ends(head_dim, theta, scaling) if hasattr(scaling, "fast") else None
     for n, i in enumerate(range(0, head_dim, 2)):
         freq = _F(1.0 / math.pow(theta, i / head_dim))
-        if scaling is not None and not hasattr(scaling, "low_freq_factor"):
+        if ends is not None:
+            ramp = min(1.0, max(0.0, (n - ends[0]) / max(ends[1] - ends[0], 0.001)))
+            freq = _F(float(freq) / scaling.factor * ramp + float(freq) * (1.0 - ramp))
+        elif scaling is not None and not hasattr(scaling, "low_freq_factor"):
             freq = _F(freq / _F(scaling.factor))          # linear scaling: every frequency divided alike
         elif scaling is not None:
             factor, lo, hi = _F(scaling.factor), _F(scaling.low_freq_factor), _F(scaling.high_freq_factor)
@@ -71,8 +89,9 @@ class Rotary:
                 freq = frequencies(spec.head_dim, spec.theta, spec.scaling)
                 pos = np.arange(spec.max_positions, dtype=_F)[:, None]
                 val = (pos * freq[None, :]).astype(_F).astype(np.float64)
-                held = _Tables(torch.from_numpy(np.cos(val).astype(_F)).to(self.device),
-                               torch.from_numpy(np.sin(val).astype(_F)).to(self.device))
+                mag = magnitude(spec.scaling)
+                held = _Tables(torch.from_numpy((mag * np.cos(val)).astype(_F)).to(self.device),
+                               torch.from_numpy((mag * np.sin(val)).astype(_F)).to(self.device))
                 Rotary._tables[key] = held
             self._held = held
         return self._held
