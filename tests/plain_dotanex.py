@@ -179,8 +179,10 @@ def dense(h, W, p):
 
 
 def expert(h, W, p, limit):
-    g = np.minimum(linear(h, W[p + "gate"]), limit)
-    u = np.clip(linear(h, W[p + "up"]), -limit, limit)
+    """``limit`` None: unbounded."""
+    g, u = linear(h, W[p + "gate"]), linear(h, W[p + "up"])
+    if limit is not None:
+        g, u = np.minimum(g, limit), np.clip(u, -limit, limit)
     return linear(g * sigmoid(1.702 * g) * (u + 1.0), W[p + "down"])
 
 
@@ -197,20 +199,25 @@ def route(h, W, p, mlp):
     return idx, w / (w.sum(-1, keepdims=True) + 1e-20), choice
 
 
-def mixture(h, W, p, mlp):
+def mixture(h, W, p, mlp, note=None):
+    """``note`` (a list) receives, per token, how far the last chosen expert's choice score lies above the first one
+    left out."""
     n_real = mlp["router"]["experts"]
-    idx, w, _ = route(h, W, p, mlp)
+    idx, w, choice = route(h, W, p, mlp)
+    if note is not None and choice.shape[-1] > mlp["router"]["top"]:
+        ranked = -np.sort(-choice, axis=-1)
+        note.extend((ranked[:, mlp["router"]["top"] - 1] - ranked[:, mlp["router"]["top"]]).tolist())
     out = np.zeros_like(h, dtype=np.float64)
     for t in range(h.shape[0]):
         for e, a in zip(idx[t], w[t]):
-            out[t] += a * (h[t] if e >= n_real else expert(h[t:t + 1], W, f"{p}e{e}.", mlp["expert"]["limit"])[0])
+            out[t] += a * (h[t] if e >= n_real else expert(h[t:t + 1], W, f"{p}e{e}.", mlp["expert"].get("limit"))[0])
     if mlp.get("shared") is not None:
-        out += expert(h, W, p + "shared.", mlp["shared"]["limit"])
+        out += expert(h, W, p + "shared.", mlp["shared"].get("limit"))
     return out
 
 
-def feed_forward(h, W, p, mlp):
-    return dense(h, W, p) if mlp["kind"] == "dense" else mixture(h, W, p, mlp)
+def feed_forward(h, W, p, mlp, note=None):
+    return dense(h, W, p) if mlp["kind"] == "dense" else mixture(h, W, p, mlp, note)
 
 
 # ----------------------------------------------------------------- the decoder
@@ -228,6 +235,7 @@ class Sequence:
         self.n = 0
         self.states = [dict() for _ in cfg["layers"]]
         self.rows = []
+        self.gaps = []          # of every router's choices so far (``mixture``)
 
     def _sublayer(self, xs, p, q, fn):
         """One sublayer under the copies' mixing: xs [T, streams, d] -> the new copies."""
@@ -257,7 +265,7 @@ class Sequence:
             if self.after:
                 self.after(i, "mixer", xs)
             if lay.get("mlp") is not None:
-                xs = self._sublayer(xs, p, 2, lambda h: feed_forward(h, W, p + "mlp.", lay["mlp"]))
+                xs = self._sublayer(xs, p, 2, lambda h: feed_forward(h, W, p + "mlp.", lay["mlp"], self.gaps))
                 if self.after:
                     self.after(i, "ffn", xs)
             rows.append(xs.sum(1))
@@ -269,3 +277,100 @@ class Sequence:
 def forward(cfg, W, tokens):
     """Logits [T, vocab] of one sequence fed whole."""
     return Sequence(cfg, W).feed(tokens)
+
+
+# ----------------------------------------------------------------- models for tests
+def tensor_shapes(cfg):
+    """Stored name -> shape of every tensor of a model of this design."""
+    d, S = cfg["width"], cfg.get("streams")
+    out = {"embed": (cfg["vocab"], d), "final.norm": (d,), "head": (cfg["vocab"], d)}
+    for i, lay in enumerate(cfg["layers"]):
+        if lay.get("weights_of") is not None:
+            continue
+        p, m, mlp = f"l{i}.", lay["mixer"], lay.get("mlp")
+        out[p + "norm1"] = (d,)
+        if S is not None:
+            out.update({p + "hc1.in": (S,), p + "hc1.mix": (S, S), p + "hc1.out": (S,)})
+        H = m["heads"]
+        if lay["type"] == "lightning":
+            out.update({p + "mix.q": (H * m["dim"], d), p + "mix.k": (H * m["dim"], d), p + "mix.v": (H * m["vdim"], d),
+                        p + "mix.g": (H * m["vdim"], d), p + "mix.o": (d, H * m["vdim"]), p + "mix.norm": (H * m["vdim"],)})
+        elif lay["type"] == "latent_attention":
+            out.update({p + "mix.dq": (m["q_rank"], d), p + "mix.dq.norm": (m["q_rank"],),
+                        p + "mix.uq": (H * (m["dim"] + m["rot_dim"]), m["q_rank"]),
+                        p + "mix.dkv": (m["kv_rank"] + m["rot_dim"], d), p + "mix.dkv.norm": (m["kv_rank"],),
+                        p + "mix.uk": (H * m["dim"], m["kv_rank"]), p + "mix.uv": (H * m["vdim"], m["kv_rank"]),
+                        p + "mix.g": (H * m["vdim"], d), p + "mix.o": (d, H * m["vdim"])})
+        else:
+            out.update({p + "mix.q": (H * m["dim"], d), p + "mix.k": (m["kv_heads"] * m["dim"], d),
+                        p + "mix.q.norm": (m["dim"],), p + "mix.k.norm": (m["dim"],), p + "mix.sink": (H,),
+                        p + "mix.o": (d, H * m["dim"])})
+        if mlp is None:
+            continue
+        out[p + "norm2"] = (d,)
+        if S is not None:
+            out.update({p + "hc2.in": (S,), p + "hc2.mix": (S, S), p + "hc2.out": (S,)})
+        q = p + "mlp."
+        if mlp["kind"] == "dense":
+            out.update({q + "gate": (mlp["ff"], d), q + "up": (mlp["ff"], d), q + "down": (d, mlp["ff"])})
+            continue
+        r = mlp["router"]
+        n_all = r["experts"] + r.get("identity", 0)
+        out.update({q + "router": (n_all, d), q + "correction": (n_all,)})
+        forms = [(f"{q}e{e}.", mlp["expert"]["ff"]) for e in range(r["experts"])]
+        if mlp.get("shared") is not None:
+            forms.append((q + "shared.", mlp["shared"]["ff"]))
+        for pre, ff in forms:
+            out.update({pre + "gate": (ff, d), pre + "up": (ff, d), pre + "down": (d, ff)})
+    return out
+
+
+def make_weights(cfg, seed):
+    """float32 weights that bfloat16 holds exactly, sized so that every mechanism moves the logits: matrices
+    N(0, 1.5/sqrt(fan-in)), norm weights around one, the copies' numbers around an even read and a kept row, sinks
+    and corrections of the size of what they stand beside."""
+    import zlib
+    import torch
+    out = {}
+    S = cfg.get("streams") or 1
+    for name, shape in tensor_shapes(cfg).items():
+        rng = np.random.default_rng([seed, zlib.crc32(name.encode())])
+        last = name.split(".")[-1]
+        if last in ("norm1", "norm2", "norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif last == "in":
+            a = 1.0 / S + 0.3 * rng.standard_normal(shape)
+        elif last == "mix":
+            a = np.eye(S) + 0.3 * rng.standard_normal(shape)
+        elif last == "out":
+            a = 1.0 + 0.3 * rng.standard_normal(shape)
+        elif last == "sink":
+            a = rng.standard_normal(shape)
+        elif last == "correction":
+            a = 0.05 * rng.standard_normal(shape)
+        else:
+            a = rng.standard_normal(shape) * (1.5 / np.sqrt(shape[-1]))
+        out[name] = torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).float().numpy()
+    return out
+
+
+def tokens_with_clear_choices(cfg, W, seed, n, gap=0.05):
+    """n token ids drawn from a seed at which no router makes a close call: at every token and layer the last chosen
+    expert's choice score lies at least ``gap`` above the first one left out, so an engine that rounds to 16 bits
+    chooses the same experts."""
+    import copy
+    rng = np.random.default_rng([seed, 11])
+    seq, out = Sequence(cfg, W), []
+    while len(out) < n:
+        for _ in range(400):
+            t = int(rng.integers(0, cfg["vocab"]))
+            trial = copy.deepcopy(seq)
+            trial.gaps, trial.rows = [], []
+            trial.feed([t])
+            if not trial.gaps or min(trial.gaps) >= gap:
+                break
+        else:
+            raise RuntimeError("no token without a close call found")
+        seq = trial
+        out.append(t)
+    return out
