@@ -31,6 +31,11 @@ state of 128, a chunked attention beside a retention, a differential attention, 
 keys and values; layer norms behind the sublayers; in every layer a routed feed-forward of 8 experts of a quarter of
 the shape's feed-forward size, two a token, beside a shared expert of that size: the shape's multiply-adds a token
 in three quarters of its feed-forward, 2.25 times its feed-forward weights).
+``--arch dotanex`` does the same for a Dotanex model (two copies of the residual row mixed around every sublayer;
+layers in turns of four: a lightning attention, an attention over cached latents, a lightning attention, a windowed
+attention with learned sinks whose values are its keys; the first layer's feed-forward is the shape's own, every other
+layer has 8 gated experts of a quarter of that size and 2 identity experts, two a token, beside a shared expert).
+``--beside nolatar`` puts a Nolatar model of the same sizes beside it instead of the Llama layers.
 """
 import argparse
 import json
@@ -115,9 +120,11 @@ def main():
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
-    ap.add_argument("--arch", default="llama", choices=["llama", "melizen", "nodupel", "nolatar"],
-                    help="melizen, nodupel, nolatar: a model of that design with the shape's sizes beside Llama layers of equal size "
-                         "(a line of its own form)")
+    ap.add_argument("--arch", default="llama", choices=["llama", "melizen", "nodupel", "nolatar", "dotanex"],
+                    help="melizen, nodupel, nolatar, dotanex: a model of that design with the shape's sizes beside Llama layers of "
+                         "equal size (a line of its own form)")
+    ap.add_argument("--beside", default="llama", choices=["llama", "melizen", "nodupel", "nolatar"],
+                    help="with --arch: the model of equal size that is measured beside it")
     ap.add_argument("--without", default="", help="names of fast paths to switch off for a comparison on the same machine, "
                     "comma-separated (parts/ops.py: tiled, packed, fused, wide, ...); the line then says so in `config`")
     args = ap.parse_args()
@@ -129,7 +136,7 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
 
-    if args.arch in ("melizen", "nodupel", "nolatar"):
+    if args.arch in ("melizen", "nodupel", "nolatar", "dotanex"):
         return other_beside_llama(args)
 
     import numpy as np
@@ -379,6 +386,32 @@ def nolatar_config(shape, layers, chunk=1024):
             "max_positions": shape["max_position_embeddings"], "layers": out}
 
 
+def dotanex_config(shape, layers, window=1024, streams=2):
+    """A Dotanex model with the sizes of a Llama shape, layers in turns of four: a lightning attention (half the
+    shape's heads, values of twice the keys' size), an attention over cached latents (the shape's heads, a rotated
+    part of half a head, latents of four heads' size for keys and values and of half the width for queries), a
+    lightning attention, and a windowed attention with the shape's heads and a sink per head. The first layer has the
+    shape's feed-forward; every other layer 8 gated experts of a quarter of its size and 2 identity experts, two a
+    token, and a shared expert of that size."""
+    d, F = shape["hidden_size"], shape["intermediate_size"]
+    H, G, hs = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    base = shape.get("rope_theta", 500000.0)
+    top = shape["max_position_embeddings"]
+    moe = {"kind": "moe", "router": {"experts": 8, "identity": 2, "top": 2}, "expert": {"ff": F // 4, "limit": 7.0},
+           "shared": {"ff": F // 4, "limit": 7.0}}
+    light = {"heads": H // 2, "dim": hs, "vdim": 2 * hs, "decay": [1.0 - 2.0 ** (-5 - (i % 8)) for i in range(H // 2)]}
+    latent = {"heads": H, "dim": hs, "rot_dim": hs // 2, "vdim": hs, "q_rank": d // 2, "kv_rank": 4 * hs,
+              "scale": (hs + hs // 2) ** -0.5,
+              "rot": {"base": base, "dims": hs // 2, "scaling": {"factor": 8.0, "original": top // 8, "fast": 32.0, "slow": 1.0}}}
+    win = {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5, "mask": {"size": window},
+           "rot": {"base": base, "dims": hs, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": top // 8}}}
+    kinds = [("lightning", light), ("latent_attention", latent), ("lightning", light), ("attention", win)]
+    out = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": F} if i == 0 else moe}
+           for i in range(layers)]
+    return {"architecture": "Dotanex", "vocab": shape["vocab_size"], "width": d, "norm": {"eps": 1e-5}, "streams": streams,
+            "max_positions": top, "layers": out}
+
+
 def other_beside_llama(args):
     """Prefill of one prompt and decode steps at --batch for a model of another design (--arch) and for Llama layers
     of equal size, one after the other on the same machine."""
@@ -394,9 +427,11 @@ def other_beside_llama(args):
     per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     arch = args.arch
-    make = {"melizen": melizen_config, "nodupel": nodupel_config, "nolatar": nolatar_config}[arch]
-    configs = {arch: g.config_from_dict(make(shape, layers)),
-               "llama": g.config_from_dict({**shape, "num_hidden_layers": layers})}
+    makers = {"melizen": melizen_config, "nodupel": nodupel_config, "nolatar": nolatar_config, "dotanex": dotanex_config}
+    beside = "llama" if args.beside == arch else args.beside
+    configs = {arch: g.config_from_dict(makers[arch](shape, layers)),
+               beside: g.config_from_dict({**shape, "num_hidden_layers": layers} if beside == "llama"
+                                          else makers[beside](shape, layers))}
     results = {}
     for name, cfg in configs.items():
         tmp = tempfile.mkdtemp(prefix="gl3-bench-")
@@ -445,7 +480,7 @@ def other_beside_llama(args):
               file=sys.stderr, flush=True)
         del eng
         torch.cuda.empty_cache()
-    m, l = results[arch], results["llama"]
+    m, l = results[arch], results[beside]
     title = arch.capitalize()
     line = {
         "metric": f"decode tok/s at batch {B}, {title} model of the {shape_name}'s sizes ({prompt_len}-token prompts)",
@@ -456,8 +491,8 @@ def other_beside_llama(args):
                    "seq_len": shape["max_position_embeddings"], "prompt_len": prompt_len, "prefill_len": prefill_len,
                    "attention_window": 1024, "parallelism": "single GPU", "sampling": "greedy on device",
                    **({"without": args.without} if args.without else {})},
-        arch: m, "llama_of_equal_size": l,
-        f"{arch}_over_llama": {"prefill_time": round(m["prefill_ms"] / l["prefill_ms"], 3),
+        arch: m, f"{beside}_of_equal_size": l,
+        f"{arch}_over_{beside}": {"prefill_time": round(m["prefill_ms"] / l["prefill_ms"], 3),
                                "decode_step_time": round(m["decode_ms_per_step"] / l["decode_ms_per_step"], 3)},
     }
     print(json.dumps(line))

@@ -1,6 +1,6 @@
 // The pieces around an attention whose keys and values are expanded from one small latent per position.
 //
-// Per position the cache keeps ONE row for all heads: [c (rank) | r (rot) | zeros up to a multiple of 16], c the
+// Per position the cache keeps ONE row for all heads: [c (rank) | r (rot) | zeros up to a multiple of 32], c the
 // normed latent and r the rotated key part that the heads share. A head's key is W_uk c beside r and its value W_uv c,
 // so with the query's unrotated part taken through W_uk^T (a row of `rank` numbers per head) the scores are dot
 // products with the cached rows themselves, and the weighted sum of the cached c goes through W_uv afterwards: the
@@ -10,6 +10,8 @@
 //                      grouped product work head by head
 //   gl3_latent_query   the rotated part of every head's query into its place behind the absorbed part
 //   gl3_sigmoid_gate   rows times the sigmoid of 32-bit gate columns
+//   gl3_latent_attention  the attention itself on the matrix cores (bfloat16; the kernel for any sizes and for 32-bit
+//                      is attention_generic.hip's, which reads values out of the key rows)
 // Norms, angles and the rotation are 32-bit arithmetic.
 #include "common.h"
 
@@ -146,6 +148,175 @@ extern "C" int gl3_sigmoid_gate(void* a, int dtype, const float* gate, long ld_g
   if (dtype == GL3_F32) sigmoid_gate_kernel<float><<<grid, block, 0, stream>>>((float*)a, gate, ld_g, col_g, C, n);
   else if (dtype == GL3_BF16) sigmoid_gate_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)a, gate, ld_g, col_g, C, n);
   else GL3_REQUIRE(false, "gl3_sigmoid_gate: unknown dtype %d", dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- the attention over the cached rows, on the matrix cores
+// q [T][H dk] (the absorbed queries), the cache rows [c | r | zeros] of dk elements (a multiple of 32), values = a
+// row's first `rank` elements (a multiple of 16). One key/value head for all query heads, so the rows of the first
+// product are (token, head) pairs: a block of NW waves takes 16 NW consecutive pairs of one sequence (row t H + h),
+// a wave 16 of them, and walks the keys 0 .. (the last pair's position) in chunks of 32 that the block stages in
+// shared memory ONCE for all its heads: as rows [key][dk] for the scores' operand, and the first `rank` columns
+// again transposed, [dim][key], for the second product's (the cache has no transposed copy of a latent).
+// Scores S = Q K^T with v_mfma_f32_16x16x32_bf16 (a lane ends up with 4 rows x 1 key of each 16 x 16 tile), scale,
+// causal mask by each pair's own position, running maximum and sum per row in 32-bit (reduced over the 16 lanes that
+// share a row), the weights in bfloat16 through a wave's own patch of shared memory into operand order, O += P V.
+// A decode step is the same kernel with one token a sequence (rows = heads).
+typedef __bf16 la_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float la_f32x4 __attribute__((ext_vector_type(4)));
+#define LA_LDV 40        // a transposed value row: 32 keys and 8 of padding
+#define LA_LDP 40        // a row of a wave's weights
+
+template <int NW, int MAXKS, int MAXDT>
+__global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
+    const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ kv_before, const int* __restrict__ block_table, const int* __restrict__ seq_rows, int table_stride,
+    bf16_t* __restrict__ out, long out_stride, int H, int dk, int rank, int page_size, float scale) {
+  extern __shared__ __attribute__((aligned(16))) char la_smem[];
+  const int s = blockIdx.y;
+  const int tok0 = cu_seqlens[s], q_len = cu_seqlens[s + 1] - tok0, before = kv_before[s];
+  const int rows_total = q_len * H;
+  const int row0 = blockIdx.x * (NW * 16);
+  if (row0 >= rows_total) return;
+  const int* bt = block_table + (long)(seq_rows ? seq_rows[s] : s) * table_stride;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
+  const int ks = dk >> 5, dt_n = rank >> 4, ldk = dk + 8;
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(la_smem);           // [32][ldk]
+  bf16_t* Vt = Ks + 32 * ldk;                                // [rank][LA_LDV]
+  bf16_t* Ps = Vt + rank * LA_LDV + wave * (16 * LA_LDP);    // [16][LA_LDP], this wave's
+  const la_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // this lane's part of the queries as the first product's operand: pair row0 + 16 wave + li, 8 elements at 32 step + 8 lq
+  const int a_row = row0 + wave * 16 + li;
+  const bool a_ok = a_row < rows_total;
+  const bf16_t* qp = q + (long)(tok0 + (a_ok ? a_row / H : 0)) * q_stride + (long)(a_ok ? a_row % H : 0) * dk + 8 * lq;
+  la_bf16x8 qf[MAXKS];
+#pragma unroll
+  for (int st = 0; st < MAXKS; ++st) qf[st] = (st < ks && a_ok) ? *reinterpret_cast<const la_bf16x8*>(qp + 32 * st) : zero;
+  // the four pairs whose sums this lane holds: rows 4 lq + i of the wave's 16
+  int pos[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + wave * 16 + 4 * lq + i;
+    pos[i] = r < rows_total ? before + r / H : -1;
+  }
+  float m_run[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l_run[4] = {0.f, 0.f, 0.f, 0.f};
+  la_f32x4 O[MAXDT];
+#pragma unroll
+  for (int dt = 0; dt < MAXDT; ++dt) O[dt] = la_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int last = (row0 + NW * 16 < rows_total ? row0 + NW * 16 : rows_total) - 1;
+  const int p_max = before + last / H;
+  const int cbs = dk >> 3, pieces = 32 * cbs;
+  for (int k0 = 0; k0 <= p_max; k0 += 32) {
+    __syncthreads();
+    // 32 keys into shared memory; piece e is 8 consecutive elements of the cache in the cache's own order
+    const bf16_t* src = k_cache + (long)bt[k0 / page_size] * page_size * dk + (long)((k0 % page_size) >> 5) * 32 * dk;
+    for (int e = threadIdx.x; e < pieces; e += NW * 64) {
+      const int tl = e / (16 * cbs), cb = (e >> 4) % cbs, row = e & 15;
+      const int p32 = ((row >> 2) << 3) | (tl << 2) | (row & 3);      // the key's place among the 32 (gl3_k_offset, inverted)
+      const la_bf16x8 v = k0 + p32 <= p_max ? *reinterpret_cast<const la_bf16x8*>(src + (long)e * 8) : zero;
+      *reinterpret_cast<la_bf16x8*>(Ks + p32 * ldk + cb * 8) = v;
+      if (cb * 8 < rank) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (cb * 8 + j < rank) Vt[(cb * 8 + j) * LA_LDV + p32] = v[j];
+      }
+    }
+    __syncthreads();
+    la_f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < MAXKS; ++st) {
+      if (st < ks) {
+        const la_bf16x8 b0 = *reinterpret_cast<const la_bf16x8*>(Ks + li * ldk + 32 * st + 8 * lq);
+        const la_bf16x8 b1 = *reinterpret_cast<const la_bf16x8*>(Ks + (16 + li) * ldk + 32 * st + 8 * lq);
+        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], b0, S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], b1, S1, 0, 0, 0);
+      }
+    }
+    float alpha[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float s0 = k0 + li <= pos[i] ? S0[i] * scale : -INFINITY;
+      const float s1 = k0 + 16 + li <= pos[i] ? S1[i] * scale : -INFINITY;
+      float mx = fmaxf(s0, s1);
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_new = fmaxf(m_run[i], mx);
+      const float p0 = s0 == -INFINITY ? 0.f : expf(s0 - m_new), p1 = s1 == -INFINITY ? 0.f : expf(s1 - m_new);
+      float rs = p0 + p1;
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o, 64);
+      alpha[i] = m_run[i] == -INFINITY ? 0.f : expf(m_run[i] - m_new);
+      l_run[i] = l_run[i] * alpha[i] + rs;
+      m_run[i] = m_new;
+      Ps[(4 * lq + i) * LA_LDP + li] = static_cast<bf16_t>(p0);
+      Ps[(4 * lq + i) * LA_LDP + 16 + li] = static_cast<bf16_t>(p1);
+    }
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[dt][i] *= alpha[i];
+    __syncthreads();                          // (the weights of this wave's rows lie in its patch)
+    const la_bf16x8 pf = *reinterpret_cast<const la_bf16x8*>(Ps + li * LA_LDP + 8 * lq);
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) {
+      if (dt < dt_n) {
+        const la_bf16x8 b = *reinterpret_cast<const la_bf16x8*>(Vt + (16 * dt + li) * LA_LDV + 8 * lq);
+        O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, b, O[dt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + wave * 16 + 4 * lq + i;
+    if (r >= rows_total) continue;
+    bf16_t* op = out + (long)(tok0 + r / H) * out_stride + (long)(r % H) * rank + li;
+    const float inv = 1.0f / l_run[i];
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt)
+      if (dt < dt_n) op[16 * dt] = static_cast<bf16_t>(O[dt][i] * inv);
+  }
+}
+
+static inline size_t la_smem_bytes(int nw, int dk, int rank) {
+  return ((size_t)32 * (dk + 8) + (size_t)rank * LA_LDV + (size_t)nw * 16 * LA_LDP) * sizeof(bf16_t);
+}
+
+// Whether the kernel is built for these sizes: cached rows of a multiple of 32 up to 288 elements, values of a multiple
+// of 16 up to 256, pages of a multiple of 32.
+extern "C" int gl3_latent_attention_supports(int dk, int rank, int page_size) {
+  return dk > 0 && dk % 32 == 0 && dk <= 288 && rank > 0 && rank % 16 == 0 && rank <= 256 && rank <= dk && page_size > 0 &&
+         page_size % 32 == 0 && la_smem_bytes(8, dk, rank) <= 64000;
+}
+
+extern "C" int gl3_latent_attention(const void* q, long q_stride, const void* k_cache, const int* cu_seqlens, const int* kv_before,
+                                    const int* block_table, const int* seq_rows, int table_stride, void* out, long out_stride,
+                                    int n_seqs, int max_q_len, int H, int dk, int rank, int page_size, float scale,
+                                    hipStream_t stream) {
+  if (n_seqs == 0 || max_q_len == 0) return 0;
+  GL3_REQUIRE(q && k_cache && cu_seqlens && kv_before && block_table && out && table_stride > 0, "gl3_latent_attention: null argument");
+  GL3_REQUIRE(gl3_latent_attention_supports(dk, rank, page_size),
+              "gl3_latent_attention: cached rows of %d with values of %d in pages of %d are not built", dk, rank, page_size);
+  GL3_REQUIRE(H > 0 && q_stride >= (long)H * dk && out_stride >= (long)H * rank && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
+                  (uintptr_t)k_cache % 16 == 0,
+              "gl3_latent_attention: rows of %ld for %d heads of %d; queries and cache 16-byte aligned", q_stride, H, dk);
+  const long rows = (long)max_q_len * H;
+  const int nw = rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+  const long blocks = (rows + nw * 16 - 1) / (nw * 16);
+  GL3_REQUIRE(blocks < (1L << 31) && n_seqs <= 65535, "gl3_latent_attention: too many blocks");
+  const dim3 grid((unsigned)blocks, n_seqs);
+  const size_t sh = la_smem_bytes(nw, dk, rank);
+  const bool small = dk <= 96 && rank <= 64;
+#define LA_GO(NW, KS, DT)                                                                                             \
+  latent_attention_kernel<NW, KS, DT><<<grid, dim3(NW * 64), sh, stream>>>(                                           \
+      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, cu_seqlens, kv_before, block_table, seq_rows, table_stride, \
+      (bf16_t*)out, out_stride, H, dk, rank, page_size, scale)
+  if (small) {
+    if (nw == 2) LA_GO(2, 3, 4); else if (nw == 4) LA_GO(4, 3, 4); else LA_GO(8, 3, 4);
+  } else {
+    if (nw == 2) LA_GO(2, 9, 16); else if (nw == 4) LA_GO(4, 9, 16); else LA_GO(8, 9, 16);
+  }
+#undef LA_GO
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -77,6 +77,8 @@ def _declare(lib):
         "gl3_latent_prep": [P, L, I, I, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, I, I, I, P, P, P],
         "gl3_latent_query": [P, I, I, I, I, I, P, P, P, P, I, I, P],
         "gl3_sigmoid_gate": [P, I, P, L, I, I, I, P],
+        "gl3_latent_attention_supports": [I, I, I],
+        "gl3_latent_attention": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
@@ -937,6 +939,39 @@ def latent_query(q, H, dim, rot, positions, cos, sin, qa, rank):
             raise KernelError(f"latent_query: table {tuple(cos.shape)} for {rot} rotated elements")
     _check(library().gl3_latent_query(_ptr(q), _code(q, "q"), T, int(H), int(dim), int(rot), _ptr(positions), _ptr(cos),
                                       _ptr(sin), _ptr(qa), int(rank), dk, _stream()), "latent_query")
+
+
+def latent_attention_fits(dk, rank, page_size):
+    """Whether the matrix-core attention over cached latents is built for rows of ``dk`` with values of ``rank``."""
+    return bool(library().gl3_latent_attention_supports(int(dk), int(rank), int(page_size)))
+
+
+def latent_attention(q, k_cache, cu_seqlens, kv_before, block_table, out, max_q_len, H, rank, scale, seq_rows=None):
+    """Causal attention of ``q`` [T, H dk] (bfloat16) over a cache of one array, ``k_cache`` [page, 1, page_size, dk],
+    whose rows are keys and, in their first ``rank`` elements, values, for all H heads alike; ``out`` [T, H rank].
+    ``cu_seqlens`` [B + 1] and ``kv_before`` [B] say which tokens of the packed ``q`` belong to which sequence and
+    where they sit in it; ``seq_rows`` [B] (optional) names each sequence's row of ``block_table``."""
+    _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
+    _dev(k_cache, "k_cache", torch.bfloat16)
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(kv_before, "kv_before", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    T, B = q.shape[0], kv_before.numel()
+    if k_cache.dim() != 4 or k_cache.shape[1] != 1:
+        raise KernelError(f"latent_attention: a cache of {tuple(k_cache.shape)}")
+    page, dk = k_cache.shape[2], k_cache.shape[3]
+    if (q.dim() != 2 or q.stride(1) != 1 or q.shape[1] != H * dk or out.shape != (T, H * rank) or out.stride(1) != 1
+            or cu_seqlens.numel() != B + 1 or block_table.dim() != 2 or max_q_len < 1):
+        raise KernelError(f"latent_attention: q {tuple(q.shape)}, out {tuple(out.shape)} for {H} heads of {dk} / {rank}")
+    if seq_rows is not None:
+        _dev(seq_rows, "seq_rows", torch.int32)
+        if seq_rows.numel() != B:
+            raise KernelError("latent_attention: one table row per sequence")
+    elif block_table.shape[0] < B:
+        raise KernelError("latent_attention: the block table has fewer rows than there are sequences")
+    _check(library().gl3_latent_attention(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(cu_seqlens), _ptr(kv_before),
+                                          _ptr(block_table), _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B,
+                                          int(max_q_len), int(H), dk, int(rank), page, float(scale), _stream()),
+           "latent_attention")
 
 
 def sigmoid_gate(a, gate, col_g):

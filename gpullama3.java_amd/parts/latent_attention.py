@@ -5,12 +5,14 @@
     key_h = [W_uk,h c | r],  value_h = W_uv,h c;   softmax((q_h . key_h) scale) over the positions so far
     output = W_o ((the heads' outputs) * sigmoid(W_g h))
 
-The cache keeps per position the row [c | r] alone (padded with zeros to a multiple of 16), for all heads together:
+The cache keeps per position the row [c | r] alone (padded with zeros to a multiple of 32), for all heads together:
 ``KVNeed(1 head, values=False)``. The heads' keys and values are never written out. Since
 ``q_h . (W_uk,h c) = (W_uk,h^T q_h) . c``, the unrotated part of a head's query is taken through ``W_uk,h^T`` into a row
 of ``kv_rank`` numbers (the grouped product of ``csrc/routed.hip``, with the heads in the experts' place), the rotated
 part is put behind it, and the attention runs over the cached rows as they are: one key head shared by all query
-heads, whose values are the keys' first ``kv_rank`` elements (``lib.attention_generic`` with ``values_in_keys``). Its
+heads, whose values are the keys' first ``kv_rank`` elements (``lib.latent_attention`` on the matrix cores, which
+stages a chunk of cached rows in shared memory once for all heads of a tile; ``lib.attention_generic`` with
+``values_in_keys`` in 32-bit and for sizes that kernel is not built for). Its
 output, the weighted sum of latents per head, goes through ``W_uv,h`` (the grouped product again), the gate and the
 output projection.
 
@@ -43,7 +45,7 @@ class LatentAttention:
             raise ValueError("the rotated key part is turned as a whole, in adjacent pairs")
         if self.R and self.position is None:
             raise ValueError("a rotated key part needs a rotation")
-        self.dk = -(-(self.rank + self.R) // 16) * 16        # a cached row, in the cache's tiles of 16
+        self.dk = -(-(self.rank + self.R) // 32) * 32        # a cached row: whole steps of the matrix cores' first product
         self.names = spec.names
         self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.off_q, self.off_kv = 0, self.q_rank
@@ -118,8 +120,13 @@ class LatentAttention:
                       mfma=mfma)
         K.latent_query(q, H, D, R, ctx.positions, cos, sin, qa, rank)
         att = ctx.buffer("latent_att", (T, H * rank), self.dtype)
-        K.attention_generic(qa, k_cache, None, ctx.positions, ops._table_rows(ctx), table, att, H, 1, dk, page, None,
-                            self.spec.scale, v_head_dim=rank, values_in_keys=0)
+        if (self.dtype == torch.bfloat16 and not ops._off(ctx) & {"attn_prefill", "attn_decode"}
+                and K.latent_attention_fits(dk, rank, page)):
+            K.latent_attention(qa, k_cache, ctx.cu_seqlens, ctx.kv_before, table, att, ctx.max_q_len, H, rank, self.spec.scale,
+                               seq_rows=getattr(ctx, "seq_rows", None))
+        else:       # (32-bit, or sizes that the matrix-core kernel is not built for)
+            K.attention_generic(qa, k_cache, None, ctx.positions, ops._table_rows(ctx), table, att, H, 1, dk, page, None,
+                                self.spec.scale, v_head_dim=rank, values_in_keys=0)
         o = ctx.buffer("latent_out", (T, H * vd), self.dtype)
         K.expert_gemm(att.view(T * H, rank), self.w_uv, o.view(T * H, vd), offsets=runs, pairs=rows, mfma=mfma)
         K.sigmoid_gate(o, proj, self.off_g)

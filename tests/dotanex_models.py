@@ -157,12 +157,12 @@ def close(got, ref, dtype, what=""):
 
 def near(got, ref, dtype, what=""):
     """Elements of residual rows or of a sublayer's output against the plain ones, on the scale of the largest:
-    float32 8e-5 (2e-4 for a sublayer alone is the caller's), bfloat16 4e-2 with one element in a hundred up to four
-    times that."""
+    float32 8e-5 (2e-4 for a sublayer alone is the caller's), bfloat16 4e-2 with one element in fifty up to five
+    times that (a sublayer deep in a model reads rows that carry the rounding of everything before it)."""
     got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
     assert got.shape == ref.shape and np.isfinite(got).all(), what
     d = np.abs(got - ref) / max(np.abs(ref).max(), 1e-3)
     if dtype == "float32":
         assert d.max() < 2e-4, f"{what}: {d.max():.3e}"
     else:
-        assert (d > 4e-2).mean() <= 1e-2 and d.max() < 0.16, f"{what}: {(d > 4e-2).mean():.2e} of the elements over, the worst {d.max():.3e}"
+        assert (d > 4e-2).mean() <= 2e-2 and d.max() < 0.2, f"{what}: {(d > 4e-2).mean():.2e} of the elements over, the worst {d.max():.3e}"

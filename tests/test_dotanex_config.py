@@ -55,7 +55,7 @@ def test_cache_needs():
     kv, state = m.cache_needs()
     assert kv[0] is None and kv[3] is None and state[0].elements == state[3].elements == 3 * 24 * 40
     assert (kv[1].n_kv_heads, kv[1].head_dim, kv[1].window, kv[1].values) == (2, 32, 37, True)       # (heads padded to 16s)
-    assert (kv[2].n_kv_heads, kv[2].head_dim, kv[2].values) == (1, 48, False) and kv[4] == kv[2]     # a latent of 40 + 8, one array
+    assert (kv[2].n_kv_heads, kv[2].head_dim, kv[2].values) == (1, 64, False) and kv[4] == kv[2]     # a latent of 40 + 8 in rows of 64, one array
     assert state[1] is None and state[2] is None
 
 

@@ -207,6 +207,41 @@ def test_values_inside_the_keys_and_a_far_marked_latent(H, rank, rot, dtype):
     assert np.median(far) > 0.5 * 40.0 / np.sqrt(rank)          # position 3 still carries the far queries' outputs
 
 
+@pytest.mark.parametrize("kind", ["decode", "prompt", "portion"])
+@pytest.mark.parametrize("H, rank, rot", [(3, 48, 16), (8, 64, 16), (16, 96, 32), (32, 256, 32), (5, 16, 4), (70, 32, 32), (1, 64, 64)])
+def test_cached_latents_on_the_matrix_cores(H, rank, rot, kind):
+    """The same attention from the matrix-core kernel: tiles of (token, head) pairs that span several tokens or a part
+    of one token's heads, one token a sequence or a portion of a prompt behind 150 cached positions, a marked latent
+    far back, keys up to the tokens' own positions and no further."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng([H, rank, 2])
+    dk = -(-(rank + rot) // 32) * 32
+    assert K.latent_attention_fits(dk, rank, 64)
+    S, at = 420, 3
+    rows = np.zeros((S, 1, dk))
+    rows[:, 0, :rank + rot] = bf16_exact(rng.standard_normal((S, rank + rot)) * 0.3)
+    rows[at, 0, :rank] = bf16_exact(40.0 / np.sqrt(rank))
+    kc, _, table = paged(rows, None, 64, "bfloat16")
+    if kind == "decode":
+        positions = [0, 2, 3, 4, 31, 32, 63, 64, 65, 127, 128, 300, S - 1]
+        cu, before, seq_rows, longest = list(range(len(positions) + 1)), positions, [0] * len(positions), 1
+    else:
+        first = 0 if kind == "prompt" else 150
+        positions = list(range(first, first + 170))
+        cu, before, seq_rows, longest = [0, len(positions)], [first], [0], len(positions)
+    T = len(positions)
+    q = np.zeros((T, H, dk))
+    q[:, :, :rank + rot] = rng.standard_normal((T, H, rank + rot)) * 0.3
+    q[:, :, :rank] += 1.0 / np.sqrt(rank)
+    q = bf16_exact(q)
+    out = torch.zeros(T, H * rank, dtype=torch.bfloat16, device=DEV)
+    K.latent_attention(dev(q.reshape(T, H * dk), torch.bfloat16), kc, i32(cu), i32(before), table, out, longest, H, rank, 0.4,
+                       seq_rows=i32(seq_rows))
+    ref = plain_heads(q, rows, rows[:, :, :rank], positions, 0.4)
+    np.testing.assert_allclose(host(out).reshape(T, H, rank), ref, atol=0.03, rtol=0.01)
+    assert np.median(ref[-1, :, 0]) > 0.5 * 40.0 / np.sqrt(rank)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, D, R, q_rank, rank", [(3, 24, 8, 48, 40), (4, 64, 32, 96, 64), (2, 16, 4, 16, 32), (5, 8, 2, 20, 24)])
 def test_latents_normed_turned_and_cached(H, D, R, q_rank, rank, dtype):
