@@ -168,118 +168,200 @@ typedef float la_f32x4 __attribute__((ext_vector_type(4)));
 #define LA_LDV 40        // a transposed value row: 32 keys and 8 of padding
 #define LA_LDP 40        // a row of a wave's weights
 
-template <int NW, int MAXKS, int MAXDT>
+template <int NW, int RT, int MAXKS, int MAXDT>
 __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const int* __restrict__ cu_seqlens,
     const int* __restrict__ kv_before, const int* __restrict__ block_table, const int* __restrict__ seq_rows, int table_stride,
-    bf16_t* __restrict__ out, long out_stride, int H, int dk, int rank, int page_size, float scale) {
+    bf16_t* __restrict__ out, long out_stride, int H, int dk, int rank, int page_size, float scale, int n_splits,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  // a wave takes RT tiles of 16 pairs: an operand of keys or values read from shared memory serves all of them
+  constexpr int MAXP = (32 * MAXKS * 4 + NW * 64 - 1) / (NW * 64);      // pieces of a chunk that a thread carries
+  constexpr int ROWS = NW * RT * 16;
   extern __shared__ __attribute__((aligned(16))) char la_smem[];
-  const int s = blockIdx.y;
+  const int s = blockIdx.y, split = blockIdx.z;
   const int tok0 = cu_seqlens[s], q_len = cu_seqlens[s + 1] - tok0, before = kv_before[s];
   const int rows_total = q_len * H;
-  const int row0 = blockIdx.x * (NW * 16);
+  const int row0 = blockIdx.x * ROWS;
   if (row0 >= rows_total) return;
   const int* bt = block_table + (long)(seq_rows ? seq_rows[s] : s) * table_stride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
   const int ks = dk >> 5, dt_n = rank >> 4, ldk = dk + 8;
-  bf16_t* Ks = reinterpret_cast<bf16_t*>(la_smem);           // [32][ldk]
-  bf16_t* Vt = Ks + 32 * ldk;                                // [rank][LA_LDV]
-  bf16_t* Ps = Vt + rank * LA_LDV + wave * (16 * LA_LDP);    // [16][LA_LDP], this wave's
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(la_smem);                 // [32][ldk]
+  bf16_t* Vt = Ks + 32 * ldk;                                      // [rank][LA_LDV]
+  bf16_t* Ps = Vt + rank * LA_LDV + wave * (RT * 16 * LA_LDP);     // [RT 16][LA_LDP], this wave's
   const la_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  // this lane's part of the queries as the first product's operand: pair row0 + 16 wave + li, 8 elements at 32 step + 8 lq
-  const int a_row = row0 + wave * 16 + li;
-  const bool a_ok = a_row < rows_total;
-  const bf16_t* qp = q + (long)(tok0 + (a_ok ? a_row / H : 0)) * q_stride + (long)(a_ok ? a_row % H : 0) * dk + 8 * lq;
-  la_bf16x8 qf[MAXKS];
+  const int wrow0 = row0 + wave * RT * 16;
+  // this lane's part of the queries as the first product's operand: pair wrow0 + 16 rt + li, 8 elements at 32 step + 8 lq
+  la_bf16x8 qf[RT][MAXKS];
+  int pos[RT][4];
+  float m_run[RT][4], l_run[RT][4];
+  la_f32x4 O[RT][MAXDT];
 #pragma unroll
-  for (int st = 0; st < MAXKS; ++st) qf[st] = (st < ks && a_ok) ? *reinterpret_cast<const la_bf16x8*>(qp + 32 * st) : zero;
-  // the four pairs whose sums this lane holds: rows 4 lq + i of the wave's 16
-  int pos[4];
+  for (int rt = 0; rt < RT; ++rt) {
+    const int a_row = wrow0 + 16 * rt + li;
+    const bool a_ok = a_row < rows_total;
+    const bf16_t* qp = q + (long)(tok0 + (a_ok ? a_row / H : 0)) * q_stride + (long)(a_ok ? a_row % H : 0) * dk + 8 * lq;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = row0 + wave * 16 + 4 * lq + i;
-    pos[i] = r < rows_total ? before + r / H : -1;
+    for (int st = 0; st < MAXKS; ++st) qf[rt][st] = (st < ks && a_ok) ? *reinterpret_cast<const la_bf16x8*>(qp + 32 * st) : zero;
+    // the four pairs whose sums this lane holds: rows 4 lq + i of the tile's 16
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = wrow0 + 16 * rt + 4 * lq + i;
+      pos[rt][i] = r < rows_total ? before + r / H : -1;
+      m_run[rt][i] = -INFINITY;
+      l_run[rt][i] = 0.f;
+    }
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) O[rt][dt] = la_f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  float m_run[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l_run[4] = {0.f, 0.f, 0.f, 0.f};
-  la_f32x4 O[MAXDT];
-#pragma unroll
-  for (int dt = 0; dt < MAXDT; ++dt) O[dt] = la_f32x4{0.f, 0.f, 0.f, 0.f};
-  const int last = (row0 + NW * 16 < rows_total ? row0 + NW * 16 : rows_total) - 1;
+  const int last = (row0 + ROWS < rows_total ? row0 + ROWS : rows_total) - 1;
   const int p_max = before + last / H;
+  // this block's share of the keys: whole chunks of 32, the splits one after another
+  const int chunks = p_max / 32 + 1, per = (chunks + n_splits - 1) / n_splits;
+  const int k_lo = split * per * 32;
+  const int k_end = (split + 1) * per * 32 - 1 < p_max ? (split + 1) * per * 32 - 1 : p_max;
   const int cbs = dk >> 3, pieces = 32 * cbs;
-  for (int k0 = 0; k0 <= p_max; k0 += 32) {
-    __syncthreads();
-    // 32 keys into shared memory; piece e is 8 consecutive elements of the cache in the cache's own order
+  // a chunk travels from memory into registers while the chunk before it is worked on; piece e is 8 consecutive
+  // elements of the cache in the cache's own order
+  la_bf16x8 pre[MAXP];
+  auto fetch = [&](int k0) {
     const bf16_t* src = k_cache + (long)bt[k0 / page_size] * page_size * dk + (long)((k0 % page_size) >> 5) * 32 * dk;
-    for (int e = threadIdx.x; e < pieces; e += NW * 64) {
-      const int tl = e / (16 * cbs), cb = (e >> 4) % cbs, row = e & 15;
-      const int p32 = ((row >> 2) << 3) | (tl << 2) | (row & 3);      // the key's place among the 32 (gl3_k_offset, inverted)
-      const la_bf16x8 v = k0 + p32 <= p_max ? *reinterpret_cast<const la_bf16x8*>(src + (long)e * 8) : zero;
-      *reinterpret_cast<la_bf16x8*>(Ks + p32 * ldk + cb * 8) = v;
-      if (cb * 8 < rank) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (cb * 8 + j < rank) Vt[(cb * 8 + j) * LA_LDV + p32] = v[j];
+    for (int u = 0; u < MAXP; ++u) {
+      const int e = threadIdx.x + u * NW * 64;
+      if (e < pieces) pre[u] = *reinterpret_cast<const la_bf16x8*>(src + (long)e * 8);
+    }
+  };
+  if (k_lo <= k_end) fetch(k_lo);
+  for (int k0 = k_lo; k0 <= k_end; k0 += 32) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MAXP; ++u) {
+      const int e = threadIdx.x + u * NW * 64;
+      if (e < pieces) {
+        const int tl = e / (16 * cbs), cb = (e >> 4) % cbs, row = e & 15;
+        const int p32 = ((row >> 2) << 3) | (tl << 2) | (row & 3);      // the key's place among the 32 (gl3_k_offset, inverted)
+        const la_bf16x8 v = k0 + p32 <= p_max ? pre[u] : zero;
+        *reinterpret_cast<la_bf16x8*>(Ks + p32 * ldk + cb * 8) = v;
+        if (cb * 8 < rank) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (cb * 8 + j < rank) Vt[(cb * 8 + j) * LA_LDV + p32] = v[j];
+        }
       }
     }
     __syncthreads();
-    la_f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
+    if (k0 + 32 <= k_end) fetch(k0 + 32);
+    la_f32x4 S0[RT], S1[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) S0[rt] = S1[rt] = la_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int st = 0; st < MAXKS; ++st) {
       if (st < ks) {
         const la_bf16x8 b0 = *reinterpret_cast<const la_bf16x8*>(Ks + li * ldk + 32 * st + 8 * lq);
         const la_bf16x8 b1 = *reinterpret_cast<const la_bf16x8*>(Ks + (16 + li) * ldk + 32 * st + 8 * lq);
-        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], b0, S0, 0, 0, 0);
-        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], b1, S1, 0, 0, 0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          S0[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[rt][st], b0, S0[rt], 0, 0, 0);
+          S1[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[rt][st], b1, S1[rt], 0, 0, 0);
+        }
       }
     }
-    float alpha[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float s0 = k0 + li <= pos[i] ? S0[i] * scale : -INFINITY;
-      const float s1 = k0 + 16 + li <= pos[i] ? S1[i] * scale : -INFINITY;
-      float mx = fmaxf(s0, s1);
+    for (int rt = 0; rt < RT; ++rt) {
+      float alpha[4];
 #pragma unroll
-      for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      const float m_new = fmaxf(m_run[i], mx);
-      const float p0 = s0 == -INFINITY ? 0.f : expf(s0 - m_new), p1 = s1 == -INFINITY ? 0.f : expf(s1 - m_new);
-      float rs = p0 + p1;
+      for (int i = 0; i < 4; ++i) {
+        const float s0 = k0 + li <= pos[rt][i] ? S0[rt][i] * scale : -INFINITY;
+        const float s1 = k0 + 16 + li <= pos[rt][i] ? S1[rt][i] * scale : -INFINITY;
+        float mx = fmaxf(s0, s1);
 #pragma unroll
-      for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o, 64);
-      alpha[i] = m_run[i] == -INFINITY ? 0.f : expf(m_run[i] - m_new);
-      l_run[i] = l_run[i] * alpha[i] + rs;
-      m_run[i] = m_new;
-      Ps[(4 * lq + i) * LA_LDP + li] = static_cast<bf16_t>(p0);
-      Ps[(4 * lq + i) * LA_LDP + 16 + li] = static_cast<bf16_t>(p1);
+        for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float m_new = fmaxf(m_run[rt][i], mx);
+        const float p0 = s0 == -INFINITY ? 0.f : expf(s0 - m_new), p1 = s1 == -INFINITY ? 0.f : expf(s1 - m_new);
+        float rs = p0 + p1;
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o, 64);
+        alpha[i] = m_run[rt][i] == -INFINITY ? 0.f : expf(m_run[rt][i] - m_new);
+        l_run[rt][i] = l_run[rt][i] * alpha[i] + rs;
+        m_run[rt][i] = m_new;
+        Ps[(16 * rt + 4 * lq + i) * LA_LDP + li] = static_cast<bf16_t>(p0);
+        Ps[(16 * rt + 4 * lq + i) * LA_LDP + 16 + li] = static_cast<bf16_t>(p1);
+      }
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) O[rt][dt][i] *= alpha[i];
     }
-#pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) O[dt][i] *= alpha[i];
     __syncthreads();                          // (the weights of this wave's rows lie in its patch)
-    const la_bf16x8 pf = *reinterpret_cast<const la_bf16x8*>(Ps + li * LA_LDP + 8 * lq);
+    la_bf16x8 pf[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) pf[rt] = *reinterpret_cast<const la_bf16x8*>(Ps + (16 * rt + li) * LA_LDP + 8 * lq);
 #pragma unroll
     for (int dt = 0; dt < MAXDT; ++dt) {
       if (dt < dt_n) {
         const la_bf16x8 b = *reinterpret_cast<const la_bf16x8*>(Vt + (16 * dt + li) * LA_LDV + 8 * lq);
-        O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, b, O[dt], 0, 0, 0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) O[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[rt], b, O[rt][dt], 0, 0, 0);
       }
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = row0 + wave * 16 + 4 * lq + i;
-    if (r >= rows_total) continue;
-    bf16_t* op = out + (long)(tok0 + r / H) * out_stride + (long)(r % H) * rank + li;
-    const float inv = 1.0f / l_run[i];
+  for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt)
-      if (dt < dt_n) op[16 * dt] = static_cast<bf16_t>(O[dt][i] * inv);
+    for (int i = 0; i < 4; ++i) {
+      const int r = wrow0 + 16 * rt + 4 * lq + i;
+      if (r >= rows_total) continue;
+      if (n_splits > 1) {
+        // this split's share as it stands: the sums under its own maximum, with that maximum and its row sum
+        const long th = (long)(tok0 + r / H) * H + r % H;
+        float* po = part_o + (th * n_splits + split) * rank + li;
+#pragma unroll
+        for (int dt = 0; dt < MAXDT; ++dt)
+          if (dt < dt_n) po[16 * dt] = O[rt][dt][i];
+        if (li == 0) {
+          part_ml[(th * n_splits + split) * 2] = m_run[rt][i];
+          part_ml[(th * n_splits + split) * 2 + 1] = l_run[rt][i];
+        }
+        continue;
+      }
+      bf16_t* op = out + (long)(tok0 + r / H) * out_stride + (long)(r % H) * rank + li;
+      const float inv = 1.0f / l_run[rt][i];
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt)
+        if (dt < dt_n) op[16 * dt] = static_cast<bf16_t>(O[rt][dt][i] * inv);
+    }
   }
 }
 
-static inline size_t la_smem_bytes(int nw, int dk, int rank) {
-  return ((size_t)32 * (dk + 8) + (size_t)rank * LA_LDV + (size_t)nw * 16 * LA_LDP) * sizeof(bf16_t);
+// The splits of one (token, head) joined; one wave, a lane a split (at most 64), then a lane a value column.
+__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part_o,
+                                                                    const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                                                    long out_stride, int H, int rank, int n_splits) {
+  const long th = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float m = lane < n_splits ? part_ml[(th * n_splits + lane) * 2] : -INFINITY;
+  const float l = lane < n_splits ? part_ml[(th * n_splits + lane) * 2 + 1] : 0.f;
+  float M = m;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+  const float f = m == -INFINITY ? 0.f : expf(m - M);
+  float L = f * l;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) L += __shfl_xor(L, o, 64);
+  const float* po = part_o + th * n_splits * rank;
+  for (int d = lane; d < rank + lane; d += 64) {      // (every lane walks along: the factors travel between lanes)
+    float acc = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+      const float fs = __shfl(f, sp, 64);
+      if (d < rank) acc = fmaf(fs, po[(long)sp * rank + d], acc);
+    }
+    if (d < rank) out[(th / H) * out_stride + (th % H) * rank + d] = static_cast<bf16_t>(acc / L);
+  }
+}
+
+static inline size_t la_smem_bytes(int tiles, int dk, int rank) {      // tiles: the block's tiles of 16 pairs
+  return ((size_t)32 * (dk + 8) + (size_t)rank * LA_LDV + (size_t)tiles * 16 * LA_LDP) * sizeof(bf16_t);
 }
 
 // Whether the kernel is built for these sizes: cached rows of a multiple of 32 up to 288 elements, values of a multiple
@@ -289,10 +371,12 @@ extern "C" int gl3_latent_attention_supports(int dk, int rank, int page_size) {
          page_size % 32 == 0 && la_smem_bytes(8, dk, rank) <= 64000;
 }
 
+// n_splits > 1 (at most 64): the keys of every sequence are shared out over that many blocks, whose parts (part_o
+// [T H][n_splits][rank], part_ml [T H][n_splits][2] floats) a second kernel joins.
 extern "C" int gl3_latent_attention(const void* q, long q_stride, const void* k_cache, const int* cu_seqlens, const int* kv_before,
                                     const int* block_table, const int* seq_rows, int table_stride, void* out, long out_stride,
-                                    int n_seqs, int max_q_len, int H, int dk, int rank, int page_size, float scale,
-                                    hipStream_t stream) {
+                                    int n_tokens, int n_seqs, int max_q_len, int H, int dk, int rank, int page_size, float scale,
+                                    int n_splits, float* part_o, float* part_ml, long part_floats, hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && cu_seqlens && kv_before && block_table && out && table_stride > 0, "gl3_latent_attention: null argument");
   GL3_REQUIRE(gl3_latent_attention_supports(dk, rank, page_size),
@@ -300,23 +384,36 @@ extern "C" int gl3_latent_attention(const void* q, long q_stride, const void* k_
   GL3_REQUIRE(H > 0 && q_stride >= (long)H * dk && out_stride >= (long)H * rank && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                   (uintptr_t)k_cache % 16 == 0,
               "gl3_latent_attention: rows of %ld for %d heads of %d; queries and cache 16-byte aligned", q_stride, H, dk);
+  GL3_REQUIRE(n_splits >= 1 && n_splits <= 64, "gl3_latent_attention: n_splits=%d", n_splits);
+  if (n_splits > 1)
+    GL3_REQUIRE(part_o && part_ml && n_tokens > 0 && part_floats >= (long)n_tokens * H * n_splits * (rank + 2),
+                "gl3_latent_attention: the splits' workspace of %ld floats is too small", part_floats);
+  // A tile of 16 pairs a wave; 4 waves where a sequence brings at most 64 pairs (the waves beyond them still carry
+  // their share of every chunk), else 8: 128 pairs a block. (Two tiles a wave, which halve the reads of shared memory
+  // per multiply-add, took 252 registers a lane and one wave a SIMD: 659 us where this takes 407, 2,048 tokens of 32
+  // heads over rows of 288.)
   const long rows = (long)max_q_len * H;
-  const int nw = rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+  const int nw = rows <= 64 ? 4 : 8;
   const long blocks = (rows + nw * 16 - 1) / (nw * 16);
   GL3_REQUIRE(blocks < (1L << 31) && n_seqs <= 65535, "gl3_latent_attention: too many blocks");
-  const dim3 grid((unsigned)blocks, n_seqs);
+  const dim3 grid((unsigned)blocks, n_seqs, n_splits);
   const size_t sh = la_smem_bytes(nw, dk, rank);
   const bool small = dk <= 96 && rank <= 64;
 #define LA_GO(NW, KS, DT)                                                                                             \
-  latent_attention_kernel<NW, KS, DT><<<grid, dim3(NW * 64), sh, stream>>>(                                           \
+  latent_attention_kernel<NW, 1, KS, DT><<<grid, dim3(NW * 64), sh, stream>>>(                                        \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, cu_seqlens, kv_before, block_table, seq_rows, table_stride, \
-      (bf16_t*)out, out_stride, H, dk, rank, page_size, scale)
+      (bf16_t*)out, out_stride, H, dk, rank, page_size, scale, n_splits, part_o, part_ml)
   if (small) {
-    if (nw == 2) LA_GO(2, 3, 4); else if (nw == 4) LA_GO(4, 3, 4); else LA_GO(8, 3, 4);
+    if (nw == 4) LA_GO(4, 3, 4); else LA_GO(8, 3, 4);
   } else {
-    if (nw == 2) LA_GO(2, 9, 16); else if (nw == 4) LA_GO(4, 9, 16); else LA_GO(8, 9, 16);
+    if (nw == 4) LA_GO(4, 9, 16); else LA_GO(8, 9, 16);
   }
 #undef LA_GO
   GL3_LAUNCH_CHECK();
+  if (n_splits > 1) {
+    latent_attention_merge_kernel<<<dim3((unsigned)((long)n_tokens * H)), dim3(64), 0, stream>>>(part_o, part_ml, (bf16_t*)out,
+                                                                                               out_stride, H, rank, n_splits);
+    GL3_LAUNCH_CHECK();
+  }
   return 0;
 }

@@ -78,7 +78,7 @@ def _declare(lib):
         "gl3_latent_query": [P, I, I, I, I, I, P, P, P, P, I, I, P],
         "gl3_sigmoid_gate": [P, I, P, L, I, I, I, P],
         "gl3_latent_attention_supports": [I, I, I],
-        "gl3_latent_attention": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
+        "gl3_latent_attention": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, P, L, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
@@ -946,11 +946,22 @@ def latent_attention_fits(dk, rank, page_size):
     return bool(library().gl3_latent_attention_supports(int(dk), int(rank), int(page_size)))
 
 
-def latent_attention(q, k_cache, cu_seqlens, kv_before, block_table, out, max_q_len, H, rank, scale, seq_rows=None):
+def latent_splits(n_seqs, max_q_len, H, kv_len):
+    """Blocks that share a sequence's cached rows in ``latent_attention``: a step of few (token, head) tiles over
+    many keys is cut until the chip has blocks, each with at least four chunks of 32 keys."""
+    rows = max_q_len * H
+    blocks = n_seqs * -(-rows // (64 if rows <= 64 else 128))      # (as the kernel's launch cuts the pairs into tiles)
+    return int(max(1, min(256 // max(blocks, 1), kv_len // 128, 32)))
+
+
+def latent_attention(q, k_cache, cu_seqlens, kv_before, block_table, out, max_q_len, H, rank, scale, seq_rows=None,
+                     n_splits=1, part_o=None, part_ml=None):
     """Causal attention of ``q`` [T, H dk] (bfloat16) over a cache of one array, ``k_cache`` [page, 1, page_size, dk],
     whose rows are keys and, in their first ``rank`` elements, values, for all H heads alike; ``out`` [T, H rank].
     ``cu_seqlens`` [B + 1] and ``kv_before`` [B] say which tokens of the packed ``q`` belong to which sequence and
-    where they sit in it; ``seq_rows`` [B] (optional) names each sequence's row of ``block_table``."""
+    where they sit in it; ``seq_rows`` [B] (optional) names each sequence's row of ``block_table``. With ``n_splits``
+    > 1 (``latent_splits``) the keys are shared out over blocks whose parts go through ``part_o`` (T H n_splits rank
+    floats) and ``part_ml`` (T H n_splits 2 floats)."""
     _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
     _dev(k_cache, "k_cache", torch.bfloat16)
     _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(kv_before, "kv_before", torch.int32)
@@ -968,9 +979,16 @@ def latent_attention(q, k_cache, cu_seqlens, kv_before, block_table, out, max_q_
             raise KernelError("latent_attention: one table row per sequence")
     elif block_table.shape[0] < B:
         raise KernelError("latent_attention: the block table has fewer rows than there are sequences")
+    floats = 0
+    if n_splits > 1:
+        _dev(part_o, "part_o", torch.float32); _dev(part_ml, "part_ml", torch.float32)
+        if part_o.numel() < T * H * n_splits * rank or part_ml.numel() < T * H * n_splits * 2:
+            raise KernelError("latent_attention: the workspace of the splits is too small")
+        floats = T * H * n_splits * (rank + 2)
     _check(library().gl3_latent_attention(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(cu_seqlens), _ptr(kv_before),
-                                          _ptr(block_table), _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B,
-                                          int(max_q_len), int(H), dk, int(rank), page, float(scale), _stream()),
+                                          _ptr(block_table), _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), T, B,
+                                          int(max_q_len), int(H), dk, int(rank), page, float(scale), int(n_splits),
+                                          _ptr(part_o), _ptr(part_ml), floats, _stream()),
            "latent_attention")
 
 

@@ -7,18 +7,23 @@
 // One kernel does both ends that meet between two sublayers: it takes the output y of the sublayer before (if any),
 // writes the new copies, and makes the input h of the sublayer behind (if any) from them, so the copies make one
 // trip to memory per sublayer. Everything is 32-bit arithmetic; h takes the activations' type. The sums run in the
-// order of s, and a row's sum of squares in an order that the width alone fixes.
+// order of s, and a row's sum of squares in an order that the width alone fixes (whatever else is in the step).
 #include "common.h"
 
 #define STREAMS_MAX 8
 
-template <typename TO>
-__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ rows, int S, int d,
-                                                            const float* __restrict__ y, const float* __restrict__ mix,
-                                                            const float* __restrict__ out_w,
-                                                            const float* __restrict__ in_w,
-                                                            const float* __restrict__ norm_w, float eps,
-                                                            TO* __restrict__ h) {
+// A block of NT threads (256 or 1024) works as 1,024 lanes, column c on lane c % 1024: a thread is R = 1024 / NT of
+// them and keeps a partial sum of squares for each, a lane's sums run over its columns one after another, the lanes'
+// over 64 at a time and then over the 16 groups in their order. So both block sizes give the same bits, and a step of
+// few tokens (a handful of blocks, each waiting for its columns' trips to memory) takes the large one.
+template <typename TO, int NT>
+__global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ rows, int S, int d,
+                                                          const float* __restrict__ y, const float* __restrict__ mix,
+                                                          const float* __restrict__ out_w,
+                                                          const float* __restrict__ in_w,
+                                                          const float* __restrict__ norm_w, float eps,
+                                                          TO* __restrict__ h) {
+  constexpr int R = 1024 / NT;
   extern __shared__ float u_row[];           // [d] the mixture that the next sublayer reads
   __shared__ float scratch[16];
   __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
@@ -30,44 +35,63 @@ __global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ r
   }
   __syncthreads();
   float* xr = rows + t * S * d;
-  float ss = 0.f;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float x[STREAMS_MAX];
+  float ss[R];
 #pragma unroll
-    for (int s = 0; s < STREAMS_MAX; ++s) x[s] = s < S ? xr[(long)s * d + c] : 0.f;
-    if (y) {
-      const float yv = y[t * d + c];
-      float nx[STREAMS_MAX];
+  for (int r = 0; r < R; ++r) ss[r] = 0.f;
+  for (int base = 0; base < d; base += 1024) {
+    float x[R][STREAMS_MAX], yv[R];
 #pragma unroll
-      for (int r = 0; r < STREAMS_MAX; ++r) {
-        if (r < S) {
-          float v = 0.f;
+    for (int r = 0; r < R; ++r) {            // (a thread's loads of one round are on their way together)
+      const int c = base + r * NT + threadIdx.x;
 #pragma unroll
-          for (int s = 0; s < STREAMS_MAX; ++s)
-            if (s < S) v = fmaf(s_mix[s * S + r], x[s], v);
-          nx[r] = fmaf(s_out[r], yv, v);
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < STREAMS_MAX; ++r)
-        if (r < S) {
-          x[r] = nx[r];
-          xr[(long)r * d + c] = nx[r];
-        }
+      for (int s = 0; s < STREAMS_MAX; ++s) x[r][s] = (s < S && c < d) ? xr[(long)s * d + c] : 0.f;
+      yv[r] = (y && c < d) ? y[t * d + c] : 0.f;
     }
-    if (in_w) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < STREAMS_MAX; ++s)
-        if (s < S) u = fmaf(s_in[s], x[s], u);
-      u_row[c] = u;
-      ss = fmaf(u, u, ss);
+    for (int r = 0; r < R; ++r) {
+      const int c = base + r * NT + threadIdx.x;
+      if (c >= d) continue;
+      if (y) {
+        float nx[STREAMS_MAX];
+#pragma unroll
+        for (int q = 0; q < STREAMS_MAX; ++q) {
+          if (q < S) {
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < STREAMS_MAX; ++s)
+              if (s < S) v = fmaf(s_mix[s * S + q], x[r][s], v);
+            nx[q] = fmaf(s_out[q], yv[r], v);
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < STREAMS_MAX; ++q)
+          if (q < S) {
+            x[r][q] = nx[q];
+            xr[(long)q * d + c] = nx[q];
+          }
+      }
+      if (in_w) {
+        float v = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s)
+          if (s < S) v = fmaf(s_in[s], x[r][s], v);
+        u_row[c] = v;
+        ss[r] = fmaf(v, v, ss[r]);
+      }
     }
   }
   if (!in_w) return;
-  ss = block_sum(ss, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
-  for (int c = threadIdx.x; c < d; c += blockDim.x) h[t * d + c] = from_f32<TO>(u_row[c] * inv * norm_w[c]);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float w = wave_sum(ss[r]);
+    if ((threadIdx.x & 63) == 0) scratch[(threadIdx.x >> 6) + (NT / 64) * r] = w;
+  }
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) total += scratch[i];
+  const float inv = 1.0f / sqrtf(total / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) h[t * d + c] = from_f32<TO>(u_row[c] * inv * norm_w[c]);
 }
 
 // y null: nothing is added and the copies stay (the first sublayer of a step). in_w null: nothing is read (behind the
@@ -82,12 +106,16 @@ extern "C" int gl3_streams_step(float* rows, int n_tokens, int S, int d, const f
   GL3_REQUIRE(y || in_w, "gl3_streams_step: nothing to do");
   const size_t sh = in_w ? (size_t)d * sizeof(float) : 0;
   GL3_REQUIRE(sh <= 64000, "gl3_streams_step: rows of %d do not fit shared memory", d);
-  const dim3 grid(n_tokens), block(256);
-  if (!in_w || h_dtype == GL3_F32)
-    streams_step_kernel<float><<<grid, block, sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (float*)h);
-  else if (h_dtype == GL3_BF16)
-    streams_step_kernel<bf16_t><<<grid, block, sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (bf16_t*)h);
-  else GL3_REQUIRE(false, "gl3_streams_step: unknown dtype %d", h_dtype);
+  const dim3 grid(n_tokens);
+  const bool few = n_tokens <= 128 && d > 256;
+#define ST_GO(TO, NT) \
+  streams_step_kernel<TO, NT><<<grid, dim3(NT), sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (TO*)h)
+  if (!in_w || h_dtype == GL3_F32) {
+    if (few) ST_GO(float, 1024); else ST_GO(float, 256);
+  } else if (h_dtype == GL3_BF16) {
+    if (few) ST_GO(bf16_t, 1024); else ST_GO(bf16_t, 256);
+  } else GL3_REQUIRE(false, "gl3_streams_step: unknown dtype %d", h_dtype);
+#undef ST_GO
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -122,8 +122,13 @@ class LatentAttention:
         att = ctx.buffer("latent_att", (T, H * rank), self.dtype)
         if (self.dtype == torch.bfloat16 and not ops._off(ctx) & {"attn_prefill", "attn_decode"}
                 and K.latent_attention_fits(dk, rank, page)):
+            splits = K.latent_splits(ctx.n_seqs, ctx.max_q_len, H, ctx.kv_len_hint)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.buffer("latent_part_o", (T, H, splits, rank), torch.float32)
+                part_ml = ctx.buffer("latent_part_ml", (T, H, splits, 2), torch.float32)
             K.latent_attention(qa, k_cache, ctx.cu_seqlens, ctx.kv_before, table, att, ctx.max_q_len, H, rank, self.spec.scale,
-                               seq_rows=getattr(ctx, "seq_rows", None))
+                               seq_rows=getattr(ctx, "seq_rows", None), n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:       # (32-bit, or sizes that the matrix-core kernel is not built for)
             K.attention_generic(qa, k_cache, None, ctx.positions, ops._table_rows(ctx), table, att, H, 1, dk, page, None,
                                 self.spec.scale, v_head_dim=rank, values_in_keys=0)

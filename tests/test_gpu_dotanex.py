@@ -74,6 +74,24 @@ def test_copies_mixed_around_a_sublayer(S, d, T, dtype):
     np.testing.assert_allclose(host(out), new.sum(1)[which], atol=2e-5)
 
 
+@pytest.mark.parametrize("d", [300, 1500, 2048, 4100])
+def test_a_row_s_bits_do_not_depend_on_the_size_of_its_step(d):
+    """A step of few tokens runs on larger blocks than one of many: the same row comes out with the same bits."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng(d)
+    S, T = 3, 200
+    xs, y = rng.standard_normal((T, S * d)).astype(np.float32), rng.standard_normal((T, d)).astype(np.float32)
+    w_in, mix, w_out = (dev(rng.standard_normal(s).astype(np.float32)) for s in ((S,), (S, S), (S,)))
+    w = dev((1 + 0.2 * rng.standard_normal(d)).astype(np.float32))
+    got = []
+    for n in (T, 5):
+        rows, h = dev(xs[:n]), torch.zeros(n, d, device=DEV)
+        K.streams_step(rows, S, y=dev(y[:n]), mix=mix, out_w=w_out, in_w=w_in, norm_w=w, eps=1e-6, h=h)
+        got.append((host(rows)[:5], host(h)[:5]))
+    np.testing.assert_array_equal(got[0][0], got[1][0])
+    np.testing.assert_array_equal(got[0][1], got[1][1])
+
+
 # ----------------------------------------------------------------- attention kernels: sinks per head, window edges
 def paged(k, v, page, dtype):
     """One sequence's keys [S, G, D] and values [S, G, Dv] (None: no value array) as a paged cache in the kernels'
@@ -207,7 +225,7 @@ def test_values_inside_the_keys_and_a_far_marked_latent(H, rank, rot, dtype):
     assert np.median(far) > 0.5 * 40.0 / np.sqrt(rank)          # position 3 still carries the far queries' outputs
 
 
-@pytest.mark.parametrize("kind", ["decode", "prompt", "portion"])
+@pytest.mark.parametrize("kind", ["decode", "decode in 5 parts", "prompt", "portion", "portion in 3 parts"])
 @pytest.mark.parametrize("H, rank, rot", [(3, 48, 16), (8, 64, 16), (16, 96, 32), (32, 256, 32), (5, 16, 4), (70, 32, 32), (1, 64, 64)])
 def test_cached_latents_on_the_matrix_cores(H, rank, rot, kind):
     """The same attention from the matrix-core kernel: tiles of (token, head) pairs that span several tokens or a part
@@ -222,6 +240,8 @@ def test_cached_latents_on_the_matrix_cores(H, rank, rot, kind):
     rows[:, 0, :rank + rot] = bf16_exact(rng.standard_normal((S, rank + rot)) * 0.3)
     rows[at, 0, :rank] = bf16_exact(40.0 / np.sqrt(rank))
     kc, _, table = paged(rows, None, 64, "bfloat16")
+    splits = int(kind.split()[2]) if " in " in kind else 1
+    kind = kind.split()[0]
     if kind == "decode":
         positions = [0, 2, 3, 4, 31, 32, 63, 64, 65, 127, 128, 300, S - 1]
         cu, before, seq_rows, longest = list(range(len(positions) + 1)), positions, [0] * len(positions), 1
@@ -235,8 +255,12 @@ def test_cached_latents_on_the_matrix_cores(H, rank, rot, kind):
     q[:, :, :rank] += 1.0 / np.sqrt(rank)
     q = bf16_exact(q)
     out = torch.zeros(T, H * rank, dtype=torch.bfloat16, device=DEV)
+    parts = {}
+    if splits > 1:       # (a split may find no key of a short sequence: its part counts for nothing)
+        parts = dict(n_splits=splits, part_o=torch.zeros(T * H * splits * rank, device=DEV),
+                     part_ml=torch.zeros(T * H * splits * 2, device=DEV))
     K.latent_attention(dev(q.reshape(T, H * dk), torch.bfloat16), kc, i32(cu), i32(before), table, out, longest, H, rank, 0.4,
-                       seq_rows=i32(seq_rows))
+                       seq_rows=i32(seq_rows), **parts)
     ref = plain_heads(q, rows, rows[:, :, :rank], positions, 0.4)
     np.testing.assert_allclose(host(out).reshape(T, H, rank), ref, atol=0.03, rtol=0.01)
     assert np.median(ref[-1, :, 0]) > 0.5 * 40.0 / np.sqrt(rank)
