@@ -388,9 +388,10 @@ def nolatar_config(shape, layers, chunk=1024):
 
 def dotanex_config(shape, layers, window=1024, streams=2):
     """A Dotanex model with the sizes of a Llama shape, layers in turns of four: a lightning attention (half the
-    shape's heads, values of twice the keys' size), an attention over cached latents (the shape's heads, a rotated
-    part of half a head, latents of four heads' size for keys and values and of half the width for queries), a
-    lightning attention, and a windowed attention with the shape's heads and a sink per head. The first layer has the
+    shape's heads, values of twice the keys' size), an attention over cached latents (the shape's heads, latents of half
+    the width for queries), a
+    lightning attention, and a windowed attention with the shape's heads and a sink per head (the latents: 256 elements
+    for keys and values, or four heads' size where that is less, beside a rotated part of 32). The first layer has the
     shape's feed-forward; every other layer 8 gated experts of a quarter of its size and 2 identity experts, two a
     token, and a shared expert of that size."""
     d, F = shape["hidden_size"], shape["intermediate_size"]
@@ -400,9 +401,10 @@ def dotanex_config(shape, layers, window=1024, streams=2):
     moe = {"kind": "moe", "router": {"experts": 8, "identity": 2, "top": 2}, "expert": {"ff": F // 4, "limit": 7.0},
            "shared": {"ff": F // 4, "limit": 7.0}}
     light = {"heads": H // 2, "dim": hs, "vdim": 2 * hs, "decay": [1.0 - 2.0 ** (-5 - (i % 8)) for i in range(H // 2)]}
-    latent = {"heads": H, "dim": hs, "rot_dim": hs // 2, "vdim": hs, "q_rank": d // 2, "kv_rank": 4 * hs,
-              "scale": (hs + hs // 2) ** -0.5,
-              "rot": {"base": base, "dims": hs // 2, "scaling": {"factor": 8.0, "original": top // 8, "fast": 32.0, "slow": 1.0}}}
+    rot_dim, kv_rank = min(hs // 2, 32), min(4 * hs, 256)      # (cached rows of 288: what the matrix-core kernel takes)
+    latent = {"heads": H, "dim": hs, "rot_dim": rot_dim, "vdim": hs, "q_rank": d // 2, "kv_rank": kv_rank,
+              "scale": (hs + rot_dim) ** -0.5,
+              "rot": {"base": base, "dims": rot_dim, "scaling": {"factor": 8.0, "original": top // 8, "fast": 32.0, "slow": 1.0}}}
     win = {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5, "mask": {"size": window},
            "rot": {"base": base, "dims": hs, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": top // 8}}}
     kinds = [("lightning", light), ("latent_attention", latent), ("lightning", light), ("attention", win)]

@@ -334,30 +334,25 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
   }
 }
 
-// The splits of one (token, head) joined; one wave, a lane a split (at most 64), then a lane a value column.
-__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part_o,
-                                                                    const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-                                                                    long out_stride, int H, int rank, int n_splits) {
+// The splits of one (token, head) joined: a thread a value column; every thread works out the splits' factors itself
+// (a few numbers that the whole block reads), and adds its column over the splits in their order.
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ part_o,
+                                                                     const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                                                     long out_stride, int H, int rank, int n_splits) {
   const long th = blockIdx.x;
-  const int lane = threadIdx.x;
-  const float m = lane < n_splits ? part_ml[(th * n_splits + lane) * 2] : -INFINITY;
-  const float l = lane < n_splits ? part_ml[(th * n_splits + lane) * 2 + 1] : 0.f;
-  float M = m;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
-  const float f = m == -INFINITY ? 0.f : expf(m - M);
-  float L = f * l;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) L += __shfl_xor(L, o, 64);
+  const int d = threadIdx.x;
+  const float* ml = part_ml + th * n_splits * 2;
+  float M = -INFINITY;
+  for (int sp = 0; sp < n_splits; ++sp) M = fmaxf(M, ml[2 * sp]);
   const float* po = part_o + th * n_splits * rank;
-  for (int d = lane; d < rank + lane; d += 64) {      // (every lane walks along: the factors travel between lanes)
-    float acc = 0.f;
-    for (int sp = 0; sp < n_splits; ++sp) {
-      const float fs = __shfl(f, sp, 64);
-      if (d < rank) acc = fmaf(fs, po[(long)sp * rank + d], acc);
-    }
-    if (d < rank) out[(th / H) * out_stride + (th % H) * rank + d] = static_cast<bf16_t>(acc / L);
+  float L = 0.f, acc = 0.f;
+  for (int sp = 0; sp < n_splits; ++sp) {
+    const float m = ml[2 * sp];
+    const float f = m == -INFINITY ? 0.f : expf(m - M);
+    L = fmaf(f, ml[2 * sp + 1], L);
+    if (d < rank) acc = fmaf(f, po[(long)sp * rank + d], acc);
   }
+  if (d < rank) out[(th / H) * out_stride + (th % H) * rank + d] = static_cast<bf16_t>(acc / L);
 }
 
 static inline size_t la_smem_bytes(int tiles, int dk, int rank) {      // tiles: the block's tiles of 16 pairs
@@ -411,8 +406,8 @@ extern "C" int gl3_latent_attention(const void* q, long q_stride, const void* k_
 #undef LA_GO
   GL3_LAUNCH_CHECK();
   if (n_splits > 1) {
-    latent_attention_merge_kernel<<<dim3((unsigned)((long)n_tokens * H)), dim3(64), 0, stream>>>(part_o, part_ml, (bf16_t*)out,
-                                                                                               out_stride, H, rank, n_splits);
+    latent_attention_merge_kernel<<<dim3((unsigned)((long)n_tokens * H)), dim3((rank + 63) / 64 * 64), 0, stream>>>(
+        part_o, part_ml, (bf16_t*)out, out_stride, H, rank, n_splits);
     GL3_LAUNCH_CHECK();
   }
   return 0;

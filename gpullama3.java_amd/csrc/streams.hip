@@ -10,7 +10,7 @@
 // order of s, and a row's sum of squares in an order that the width alone fixes (whatever else is in the step).
 #include "common.h"
 
-#define STREAMS_MAX 8
+#define STREAMS_MAX 16
 
 // A block of NT threads (256 or 1024) works as 1,024 lanes, column c on lane c % 1024: a thread is R = 1024 / NT of
 // them and keeps a partial sum of squares for each, a lane's sums run over its columns one after another, the lanes'

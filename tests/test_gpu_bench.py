@@ -77,7 +77,7 @@ def test_bench_batch_64_and_a_prefill_of_8192_with_the_8b_layers():
     assert d["prefill"]["tokens"] == 8192 and d["points"] == {}
 
 
-@pytest.mark.parametrize("arch", ["melizen", "nodupel"])
+@pytest.mark.parametrize("arch", ["melizen", "nodupel", "dotanex"])
 def test_bench_another_design_beside_llama_layers_of_equal_size(arch):
     """``--arch melizen`` / ``--arch nodupel``: one line of the same outer form, with both models' prefill and decode
     and their ratio."""

@@ -40,7 +40,7 @@ def bf16_exact(a):
 
 # ----------------------------------------------------------------- the copies of the residual row
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("S, d, T", [(1, 40, 3), (2, 96, 7), (3, 256, 70), (4, 1500, 5), (8, 64, 2)])
+@pytest.mark.parametrize("S, d, T", [(1, 40, 3), (2, 96, 7), (3, 256, 70), (4, 1500, 5), (8, 64, 2), (16, 130, 3)])
 def test_copies_mixed_around_a_sublayer(S, d, T, dtype):
     from gpullama3_java_amd.csrc import lib as K
     rng = np.random.default_rng([S, d])
