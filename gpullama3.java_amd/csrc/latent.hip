@@ -165,6 +165,24 @@ extern "C" int gl3_sigmoid_gate(void* a, int dtype, const float* gate, long ld_g
 // A decode step is the same kernel with one token a sequence (rows = heads).
 typedef __bf16 la_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float la_f32x4 __attribute__((ext_vector_type(4)));
+// A value over the 16 lanes that share a row of sums (a row of the data-parallel moves): neighbours in a quad, the
+// other quad of a half, the other half; the moves are vector instructions, where a shuffle goes through shared memory.
+template <int CTRL>
+__device__ __forceinline__ float la_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float la_max16(float v) {
+  v = fmaxf(v, la_move<0xB1>(v));       // lanes 1 0 3 2 of a quad
+  v = fmaxf(v, la_move<0x4E>(v));       // lanes 2 3 0 1
+  v = fmaxf(v, la_move<0x141>(v));      // a half of 8 mirrored: the other quad's (equal) values
+  return fmaxf(v, la_move<0x140>(v));   // the row of 16 mirrored: the other half's
+}
+__device__ __forceinline__ float la_sum16(float v) {
+  v += la_move<0xB1>(v);
+  v += la_move<0x4E>(v);
+  v += la_move<0x141>(v);
+  return v + la_move<0x140>(v);
+}
 #define LA_LDV 40        // a transposed value row: 32 keys and 8 of padding
 #define LA_LDP 40        // a row of a wave's weights
 
@@ -181,8 +199,13 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
   const int s = blockIdx.y, split = blockIdx.z;
   const int tok0 = cu_seqlens[s], q_len = cu_seqlens[s + 1] - tok0, before = kv_before[s];
   const int rows_total = q_len * H;
-  const int row0 = blockIdx.x * ROWS;
-  if (row0 >= rows_total) return;
+  // A tile late in a sequence walks many keys, an early one few, and the blocks of a launch mostly run side by side:
+  // the second half of the blocks takes the tiles from the end, so that blocks which share a CU (one of each half,
+  // as blocks are handed out in order) carry about the same work together.
+  const int nb = gridDim.x, hb = (nb + 1) / 2;
+  const int tile = (int)blockIdx.x < hb ? 2 * blockIdx.x : 2 * (nb - 1 - blockIdx.x) + 1;
+  const int row0 = (tile < nb ? tile : nb - 1) * ROWS;
+  if (tile >= nb || row0 >= rows_total) return;
   const int* bt = block_table + (long)(seq_rows ? seq_rows[s] : s) * table_stride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 15, lq = lane >> 4;
   const int ks = dk >> 5, dt_n = rank >> 4, ldk = dk + 8;
@@ -221,6 +244,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
   const int k_lo = split * per * 32;
   const int k_end = (split + 1) * per * 32 - 1 < p_max ? (split + 1) * per * 32 - 1 : p_max;
   const int cbs = dk >> 3, pieces = 32 * cbs;
+  const float scale2 = scale * 1.4426950408889634f;
   // a chunk travels from memory into registers while the chunk before it is worked on; piece e is 8 consecutive
   // elements of the cache in the cache's own order
   la_bf16x8 pre[MAXP];
@@ -228,8 +252,9 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
     const bf16_t* src = k_cache + (long)bt[k0 / page_size] * page_size * dk + (long)((k0 % page_size) >> 5) * 32 * dk;
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
-      const int e = threadIdx.x + u * NW * 64;
-      if (e < pieces) pre[u] = *reinterpret_cast<const la_bf16x8*>(src + (long)e * 8);
+      const int g = threadIdx.x + u * NW * 64;      // 16 lanes a (column block, tile of 16 keys): see the staging below
+      const int e = ((g >> 4) & 1) * 16 * cbs + (g >> 5) * 16 + (g & 15);
+      if (g < pieces) pre[u] = *reinterpret_cast<const la_bf16x8*>(src + (long)e * 8);
     }
   };
   if (k_lo <= k_end) fetch(k_lo);
@@ -237,9 +262,11 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
-      const int e = threadIdx.x + u * NW * 64;
-      if (e < pieces) {
-        const int tl = e / (16 * cbs), cb = (e >> 4) % cbs, row = e & 15;
+      // (the two tiles of a column block side by side in a wave: their transposed writes fall on banks of their own,
+      // where four column blocks of one tile would share theirs)
+      const int g = threadIdx.x + u * NW * 64;
+      if (g < pieces) {
+        const int tl = (g >> 4) & 1, cb = g >> 5, row = g & 15;
         const int p32 = ((row >> 2) << 3) | (tl << 2) | (row & 3);      // the key's place among the 32 (gl3_k_offset, inverted)
         const la_bf16x8 v = k0 + p32 <= p_max ? pre[u] : zero;
         *reinterpret_cast<la_bf16x8*>(Ks + p32 * ldk + cb * 8) = v;
@@ -272,28 +299,31 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
       float alpha[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float s0 = k0 + li <= pos[rt][i] ? S0[rt][i] * scale : -INFINITY;
-        const float s1 = k0 + 16 + li <= pos[rt][i] ? S1[rt][i] * scale : -INFINITY;
-        float mx = fmaxf(s0, s1);
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        const float m_new = fmaxf(m_run[rt][i], mx);
-        const float p0 = s0 == -INFINITY ? 0.f : expf(s0 - m_new), p1 = s1 == -INFINITY ? 0.f : expf(s1 - m_new);
-        float rs = p0 + p1;
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o, 64);
-        alpha[i] = m_run[rt][i] == -INFINITY ? 0.f : expf(m_run[rt][i] - m_new);
+        // (scores in units of ln 2: the weights are powers of two, one instruction each)
+        const float s0 = k0 + li <= pos[rt][i] ? S0[rt][i] * scale2 : -INFINITY;
+        const float s1 = k0 + 16 + li <= pos[rt][i] ? S1[rt][i] * scale2 : -INFINITY;
+        const float m_new = fmaxf(m_run[rt][i], la_max16(fmaxf(s0, s1)));
+        const float p0 = s0 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s0 - m_new);
+        const float p1 = s1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s1 - m_new);
+        const float rs = la_sum16(p0 + p1);
+        alpha[i] = m_run[rt][i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[rt][i] - m_new);
         l_run[rt][i] = l_run[rt][i] * alpha[i] + rs;
         m_run[rt][i] = m_new;
         Ps[(16 * rt + 4 * lq + i) * LA_LDP + li] = static_cast<bf16_t>(p0);
         Ps[(16 * rt + 4 * lq + i) * LA_LDP + 16 + li] = static_cast<bf16_t>(p1);
       }
+      // (the sums so far shrink only when a row's maximum has grown: rarely, once a row has seen some keys)
+      if (__any(alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f)) {
 #pragma unroll
-      for (int dt = 0; dt < MAXDT; ++dt)
+        for (int dt = 0; dt < MAXDT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) O[rt][dt][i] *= alpha[i];
+          for (int i = 0; i < 4; ++i) O[rt][dt][i] *= alpha[i];
+      }
     }
-    __syncthreads();                          // (the weights of this wave's rows lie in its patch)
+    // (the weights of this wave's rows lie in its own patch: the wave's reads follow its writes in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     la_bf16x8 pf[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pf[rt] = *reinterpret_cast<const la_bf16x8*>(Ps + (16 * rt + li) * LA_LDP + 8 * lq);
@@ -320,7 +350,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attention_kernel(
         for (int dt = 0; dt < MAXDT; ++dt)
           if (dt < dt_n) po[16 * dt] = O[rt][dt][i];
         if (li == 0) {
-          part_ml[(th * n_splits + split) * 2] = m_run[rt][i];
+          part_ml[(th * n_splits + split) * 2] = m_run[rt][i] * 0.6931471805599453f;      // (as a natural logarithm)
           part_ml[(th * n_splits + split) * 2 + 1] = l_run[rt][i];
         }
         continue;

@@ -83,7 +83,7 @@ PLAIN = {
 # head sizes that the matrix cores' kernels are built for, widths in whole tiles: what a bfloat16 engine runs on its
 # fast paths (windowed attention with heads of 64 and 128, experts' products on the matrix cores); four copies
 TILED = {
-    "architecture": "Dotanex", "vocab": 640, "width": 128, "norm": {"eps": 1e-5}, "streams": 4,
+    "architecture": "Dotanex", "vocab": 704, "width": 128, "norm": {"eps": 1e-5}, "streams": 4,
     "layers": [_window(4, 2, 64, 0.125, 10000.0, 32, (8.0, 1.0, 4.0, 128), 100, _moe(8, 2, 2, 64, 2.0, (128, 1.0))),
                _lightning(4, 32, 64, [0.7, 0.9, 0.97, 0.995], _dense(256)),
                _latent(4, 64, 32, 64, 96, 64, 0.1, 40000.0, (8.0, 128, 32.0, 1.0), _moe(4, 4, 2, 64, 2.0, (64, 2.0))),
