@@ -15,8 +15,9 @@
 // A block of NT threads (256 or 1024) works as 1,024 lanes, column c on lane c % 1024: a thread is R = 1024 / NT of
 // them and keeps a partial sum of squares for each, a lane's sums run over its columns one after another, the lanes'
 // over 64 at a time and then over the 16 groups in their order. So both block sizes give the same bits, and a step of
-// few tokens (a handful of blocks, each waiting for its columns' trips to memory) takes the large one.
-template <typename TO, int NT>
+// few tokens (a handful of blocks, each waiting for its columns' trips to memory) takes the large one. MAXS bounds the
+// copies that a thread keeps in registers (4 for the usual counts: 64 registers where 16 take 100).
+template <typename TO, int NT, int MAXS>
 __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ rows, int S, int d,
                                                           const float* __restrict__ y, const float* __restrict__ mix,
                                                           const float* __restrict__ out_w,
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ ro
   constexpr int R = 1024 / NT;
   extern __shared__ float u_row[];           // [d] the mixture that the next sublayer reads
   __shared__ float scratch[16];
-  __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
+  __shared__ float s_mix[MAXS * MAXS], s_out[MAXS], s_in[MAXS];
   const long t = blockIdx.x;
   if (threadIdx.x < S * S && y) s_mix[threadIdx.x] = mix[threadIdx.x];
   if (threadIdx.x < S) {
@@ -39,12 +40,12 @@ __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ ro
 #pragma unroll
   for (int r = 0; r < R; ++r) ss[r] = 0.f;
   for (int base = 0; base < d; base += 1024) {
-    float x[R][STREAMS_MAX], yv[R];
+    float x[R][MAXS], yv[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {            // (a thread's loads of one round are on their way together)
       const int c = base + r * NT + threadIdx.x;
 #pragma unroll
-      for (int s = 0; s < STREAMS_MAX; ++s) x[r][s] = (s < S && c < d) ? xr[(long)s * d + c] : 0.f;
+      for (int s = 0; s < MAXS; ++s) x[r][s] = (s < S && c < d) ? xr[(long)s * d + c] : 0.f;
       yv[r] = (y && c < d) ? y[t * d + c] : 0.f;
     }
 #pragma unroll
@@ -52,19 +53,19 @@ __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ ro
       const int c = base + r * NT + threadIdx.x;
       if (c >= d) continue;
       if (y) {
-        float nx[STREAMS_MAX];
+        float nx[MAXS];
 #pragma unroll
-        for (int q = 0; q < STREAMS_MAX; ++q) {
+        for (int q = 0; q < MAXS; ++q) {
           if (q < S) {
             float v = 0.f;
 #pragma unroll
-            for (int s = 0; s < STREAMS_MAX; ++s)
+            for (int s = 0; s < MAXS; ++s)
               if (s < S) v = fmaf(s_mix[s * S + q], x[r][s], v);
             nx[q] = fmaf(s_out[q], yv[r], v);
           }
         }
 #pragma unroll
-        for (int q = 0; q < STREAMS_MAX; ++q)
+        for (int q = 0; q < MAXS; ++q)
           if (q < S) {
             x[r][q] = nx[q];
             xr[(long)q * d + c] = nx[q];
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ ro
       if (in_w) {
         float v = 0.f;
 #pragma unroll
-        for (int s = 0; s < STREAMS_MAX; ++s)
+        for (int s = 0; s < MAXS; ++s)
           if (s < S) v = fmaf(s_in[s], x[r][s], v);
         u_row[c] = v;
         ss[r] = fmaf(v, v, ss[r]);
@@ -108,8 +109,12 @@ extern "C" int gl3_streams_step(float* rows, int n_tokens, int S, int d, const f
   GL3_REQUIRE(sh <= 64000, "gl3_streams_step: rows of %d do not fit shared memory", d);
   const dim3 grid(n_tokens);
   const bool few = n_tokens <= 128 && d > 256;
-#define ST_GO(TO, NT) \
-  streams_step_kernel<TO, NT><<<grid, dim3(NT), sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (TO*)h)
+#define ST_GO(TO, NT)                                                                                                   \
+  do {                                                                                                                  \
+    if (S <= 4) streams_step_kernel<TO, NT, 4><<<grid, dim3(NT), sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps, (TO*)h); \
+    else streams_step_kernel<TO, NT, STREAMS_MAX><<<grid, dim3(NT), sh, stream>>>(rows, S, d, y, mix, out_w, in_w, norm_w, eps,      \
+                                                                                  (TO*)h);                              \
+  } while (0)
   if (!in_w || h_dtype == GL3_F32) {
     if (few) ST_GO(float, 1024); else ST_GO(float, 256);
   } else if (h_dtype == GL3_BF16) {
