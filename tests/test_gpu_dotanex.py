@@ -668,3 +668,96 @@ def test_the_trace_runner_replays_a_model_of_this_design(tmp_path):
     close(np.concatenate(got["c"]), ref["c"], "float32", "the shorter of a batch")
     close(np.concatenate(got["a"]), ref["a"][69:90], "float32", "the longer of a batch")
     rp.close()
+
+
+# ----------------------------------------------------------------- seeded random configurations
+def random_config(seed):
+    """A configuration drawn from a seed: copies, widths, head counts and sizes (multiples of 8 that no tile need
+    divide, latents of any even size), layer order, windows, limits, experts and identity experts, scalings on and
+    off, layers that run another layer's weights."""
+    from dotanex_models import _dense, _latent, _lightning, _moe, _window
+    rng = np.random.default_rng([seed, 77])
+    pick = lambda *a: a[int(rng.integers(0, len(a)))]
+    width = int(pick(48, 64, 72, 104, 128))
+
+    def mlp():
+        kind = pick("dense", "moe", "moe", None)
+        if kind is None:
+            return None
+        if kind == "dense":
+            return _dense(int(pick(24, 40, 56, 96)))
+        experts, identity = int(pick(1, 2, 3, 5, 8)), int(pick(0, 0, 1, 3))
+        top = int(rng.integers(1, min(experts + identity, 4) + 1))
+        shared = pick(None, (int(pick(16, 24, 40)), pick(None, 0.5, 1.0, 3.0)))
+        return _moe(experts, identity, top, int(pick(8, 24, 33, 40)), pick(None, 0.7, 1.0, 2.0), shared)
+
+    def layer():
+        kind = pick("lightning", "latent", "window")
+        if kind == "lightning":
+            H = int(pick(1, 2, 3, 5))
+            return _lightning(H, int(pick(8, 16, 20, 32)), int(pick(8, 24, 40, 64)), [float(rng.uniform(0.3, 0.9995)) for _ in range(H)], mlp())
+        if kind == "latent":
+            rot = int(pick(2, 4, 8, 16))
+            scaling = pick(None, (float(pick(2.0, 8.0, 40.0)), int(pick(16, 64, 256)), float(pick(8.0, 32.0)), float(pick(1.0, 2.0))))
+            dim = int(pick(8, 16, 24, 40))
+            return _latent(int(pick(1, 2, 3, 6)), dim, rot, int(pick(8, 16, 24, 48)), int(pick(12, 16, 40, 64)), int(pick(10, 16, 32, 48, 80)),
+                           float((dim + rot) ** -0.5 * rng.uniform(0.7, 1.4)), float(pick(100.0, 1e4, 2.5e5)), scaling, mlp())
+        G = int(pick(1, 2, 3))
+        dim = int(pick(8, 16, 24, 32, 64))
+        dims = int(pick(2, 4, 8, dim))
+        dims = min(dims, dim) // 2 * 2
+        scaling = pick(None, (float(pick(2.0, 8.0, 32.0)), 1.0, float(pick(2.0, 4.0)), int(pick(16, 64, 512))))
+        return _window(G * int(pick(1, 2, 4)), G, dim, float(dim ** -0.5 * rng.uniform(0.7, 1.4)), float(pick(100.0, 1e4, 5e5)), dims, scaling,
+                       pick(None, 1, 2, 7, 33, 64, 65, 100), mlp())
+
+    layers = [layer() for _ in range(int(rng.integers(2, 6)))]
+    for i in range(len(layers)):                        # some layers run another layer's weights
+        j = int(rng.integers(0, len(layers)))
+        if rng.random() < 0.3 and j != i and "weights_of" not in layers[j] and "weights_of" not in layers[i] \
+                and not any(l.get("weights_of") == i for l in layers):
+            layers[i] = dict(layers[j], weights_of=j)
+    cfg = {"architecture": "Dotanex", "vocab": int(pick(97, 150, 256, 301)), "width": width, "norm": {"eps": float(pick(1e-6, 1e-5))},
+           "layers": layers}
+    streams = pick(None, 1, 2, 3, 5)
+    if streams is not None:
+        cfg["streams"] = int(streams)
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_seeded_random_configurations(seed, tmp_path):
+    """Whole, in portions with the last tokens one by one, and as one of a batch of three: 32-bit against the plain
+    implementation to rounding, bfloat16 within its bound."""
+    from dotanex_models import write_model
+    from gpullama3_java_amd.engine import Engine
+    cfg = random_config(seed)
+    W = P.make_weights(cfg, seed)
+    folder = str(tmp_path / "model")
+    write_model(folder, cfg, W)
+    toks = P.tokens_with_clear_choices(cfg, W, seed, 150)
+    others = [P.tokens_with_clear_choices(cfg, W, seed + 100 + i, n) for i, n in enumerate((40, 9))]
+    ref = P.forward(cfg, W, toks)
+    refs = [P.forward(cfg, W, t) for t in others]
+    for dtype in DTYPES:
+        eng = Engine.from_folder(folder, dtype=dtype, max_tokens=1024, n_slots=4)
+        s = eng.take_slot()
+        what = f"seed {seed} {dtype}"
+        close(eng.step([(s, toks)], want="all").cpu().numpy(), ref, dtype, what + " whole", few_far=4)
+        eng.give_back_slot(s)
+        s = eng.take_slot()
+        rows = [eng.step([(s, toks[:70])], want="all").cpu().numpy(), eng.step([(s, toks[70:72])], want="all").cpu().numpy(),
+                eng.step([(s, toks[72:140])], want="all").cpu().numpy()]
+        rows += [eng.step([(s, [t])]).cpu().numpy() for t in toks[140:]]
+        close(np.concatenate(rows), ref, dtype, what + " in portions", few_far=4)
+        eng.give_back_slot(s)
+        slots = [eng.take_slot() for _ in range(3)]
+        got = eng.step([(slots[0], others[0][:30]), (slots[1], toks[:100]), (slots[2], others[1][:3])], want="all").cpu().numpy()
+        close(got[:30], refs[0][:30], dtype, what + " batch 0", few_far=2)
+        close(got[30:130], ref[:100], dtype, what + " batch 1", few_far=3)
+        close(got[130:], refs[1][:3], dtype, what + " batch 2", few_far=1)
+        for j in range(6):
+            got = eng.step([(slots[0], [others[0][30 + j]]), (slots[1], [toks[100 + j]]), (slots[2], [others[1][3 + j]])]).cpu().numpy()
+            close(got[0:1], refs[0][30 + j:31 + j], dtype, what + f" decode 0 step {j}")
+            close(got[1:2], ref[100 + j:101 + j], dtype, what + f" decode 1 step {j}")
+            close(got[2:3], refs[1][3 + j:4 + j], dtype, what + f" decode 2 step {j}")
+        del eng
