@@ -95,7 +95,9 @@ def _check_mixer(kind, m, where):
     if not isinstance(m, dict):
         raise ConfigError(f"config.json: {where}'mixer' must be an object")
     heads = _int(m, "heads", where)
-    _int(m, "dim", where), _int(m, "vdim", where)
+    _int(m, "dim", where)
+    if kind != "attention" or m.get("vdim") is not None:      # (the windowed attention's values are its keys: their size is the keys')
+        _int(m, "vdim", where)
     if kind == "lightning":
         decay = m.get("decay")
         if not isinstance(decay, list) or len(decay) != heads or any(
@@ -111,7 +113,7 @@ def _check_mixer(kind, m, where):
         kv = _int(m, "kv_heads", where)
         if heads % kv:
             raise ConfigError(f"config.json: {where}{heads} heads are not a multiple of {kv} kv_heads")
-        if m["vdim"] != m["dim"]:
+        if m.get("vdim") is not None and m["vdim"] != m["dim"]:
             raise ConfigError(f"config.json: {where}the values are the keys: 'vdim' {m['vdim']} must equal 'dim' {m['dim']}")
         _positive(m, "scale", where)
         _rot(m, m["dim"], where, ("factor", "low", "high", "original"))
